@@ -1,0 +1,131 @@
+/* awq_mi355x.h -- C ABI of libawq_mi355x.so: the AWQ W4A16 linear path for AMD MI355X
+ * (gfx950), hand-written HIP kernels behind plain pointers and sizes.
+ *
+ * What it replaces.  The benchmark harness starts a vLLM OpenAI server
+ * (reference utils/generate_compose.py:67 image, :85-93 server command) on AWQ checkpoints
+ * (reference config.yaml:36,47,51,134); every quantised Linear / fused-MoE layer of that
+ * server runs awq_dequantize / awq_gemm / the expert-grouped AWQ GEMM.  That code lives in
+ * the docker image, not in the harness repository, so each entry point below cites the
+ * harness call site that makes it run plus the operator name it stands in for.
+ *
+ * Conventions
+ *   - All pointers are DEVICE pointers (HIP), row-major, densely packed.
+ *   - AutoAWQ "GEMM" layout: qweight int32 [K, N/8], qzeros int32 [K/G, N/8],
+ *     scales fp16 [K/G, N]; nibble i of a word at word-column c holds logical column
+ *     8c + {0,2,4,6,1,3,5,7}[i].  W[k,n] = fp16((w - z) * s), one rounding.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *   - Every call validates on the host first and launches nothing on error; calls are
+ *     asynchronous, never synchronise, never allocate and never keep a pointer.
+ *   - Return value: AWQMI_OK or one of the awqmi_status codes below.
+ */
+#ifndef AWQ_MI355X_H
+#define AWQ_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum awqmi_status {
+  AWQMI_OK = 0,
+  AWQMI_BAD_SHAPE = 1,           /* M/K/N/group relations violated                        */
+  AWQMI_BAD_ALIGN = 2,           /* a pointer is not 16-byte aligned                      */
+  AWQMI_WORKSPACE_TOO_SMALL = 3, /* workspace_bytes < awqmi_*_workspace_bytes(...)        */
+  AWQMI_UNSUPPORTED_GROUP = 4,   /* group size the kernels do not cover                   */
+  AWQMI_LAUNCH_FAILED = 5,       /* hipGetLastError() != 0, see awqmi_last_hip_error()    */
+  AWQMI_NULL_POINTER = 6,
+  AWQMI_BAD_ARGUMENT = 7         /* split_k / tile_m / topk / variant out of range        */
+} awqmi_status;
+
+#define AWQMI_VERSION 100        /* major*10000 + minor*100 + patch */
+#define AWQMI_MOE_TILE_M 16      /* rows per sorted-token block the grouped GEMM consumes  */
+#define AWQMI_MAX_SPLIT_K 64
+#define AWQMI_MAX_EXPERTS 1024
+
+int awqmi_version(void);
+const char* awqmi_status_string(int status);
+/* hipError_t of the last AWQMI_LAUNCH_FAILED on the calling thread (0 if none). */
+int awqmi_last_hip_error(void);
+
+/* awq_dequantize(qweight, scales, zeros, split_k_iters, thx, thy) -> fp16 [K, N].
+ * Stands in for vLLM's `awq_dequantize` op (taken by AWQLinearMethod.apply for large M);
+ * reached from the server started at reference utils/generate_compose.py:85-93.
+ * Any group with K % group == 0; N % 8 == 0.  Bit-exact fp16((w - z) * s). */
+int awqmi_dequantize_f16(const int32_t* qweight, const void* scales_f16, const int32_t* qzeros,
+                         void* out_f16, int K, int N, int group, void* stream);
+
+/* Split-K factor the library would pick for this shape (>= 1). */
+int awqmi_gemm_auto_split_k(int M, int K, int N, int group);
+
+/* Bytes of workspace awqmi_gemm_f16 needs for this call (split_k == 0 means "auto").
+ * The first AWQMI_WS_COUNTER_BYTES of the workspace are split-K arrival counters: they
+ * must be zero before the first call and every call leaves them zero again, so one
+ * zero-initialised buffer can be reused call after call on one stream.  Two calls that
+ * overlap in time (different streams) need different workspaces. */
+#define AWQMI_WS_COUNTER_BYTES 65536
+size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k);
+
+/* awq_gemm(input, qweight, scales, qzeros, split_k_iters) -> fp16 [M, N] = X @ W.
+ * Stands in for vLLM's `awq_gemm` op (every AWQ Linear at decode and prefill); reached
+ * from the server started at reference utils/generate_compose.py:85-93.
+ * fp32 accumulation, one final rounding to fp16.  M >= 1; K % group == 0; N % 8 == 0.
+ * M <= 16 takes the HBM-bound skinny kernel (split_k honoured, 0 = auto), larger M the
+ * LDS-dequant MFMA kernel (split_k ignored).  Shapes outside the fast kernels' tiling
+ * (K % 128 != 0, group not in {32, 64, 128*i}) take a slow generic kernel. */
+int awqmi_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
+                   const int32_t* qzeros, void* y_f16, void* workspace, size_t workspace_bytes,
+                   int M, int K, int N, int group, int split_k, void* stream);
+
+/* Router: softmax over E experts, top-k (ties: lowest expert id), optional renormalise.
+ * Stands in for the fused-MoE routing step of the MoE AWQ models at reference
+ * config.yaml:36,51,134.  logits fp32 [T, E]; ids int32 [T, topk]; weights fp32 [T, topk]. */
+int awqmi_moe_topk_softmax_f32(const float* logits, int T, int E, int topk, int renormalize,
+                               int32_t* topk_ids, float* topk_weights, void* stream);
+
+/* Capacity (entries) of sorted_token_ids for n = T*topk routed slots; expert_ids needs
+ * capacity / tile_m entries. */
+size_t awqmi_moe_align_capacity(int n_slots, int E, int tile_m);
+
+/* Stable sort of the flat (token, slot) indices by expert; each expert's run is padded to a
+ * multiple of tile_m with the sentinel n_slots.  sorted_token_ids[capacity] (tail filled
+ * with the sentinel), expert_ids[capacity / tile_m] (tail filled with -1),
+ * num_tokens_post_padded[1].  Stands in for the align/sort step of fused MoE (same models).
+ * Ids outside [0, E) are dropped (they appear nowhere in the output).  E <= 1024. */
+int awqmi_moe_align(const int32_t* topk_ids, int n_slots, int E, int tile_m,
+                    int32_t* sorted_token_ids, int32_t* expert_ids,
+                    int32_t* num_tokens_post_padded, void* stream);
+
+/* Workspace bytes of one grouped GEMM call (same counter rule as awqmi_gemm_f16). */
+size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int split_k);
+
+/* Expert-grouped AWQ GEMM over sorted-token blocks of AWQMI_MOE_TILE_M rows.
+ * For every non-pad entry s = sorted_token_ids[i] in a block owned by expert e:
+ *     y[s, :] = (x[s / a_row_div, :] @ W_e) * (topk_weights ? topk_weights[s] : 1)
+ * a_row_div = topk for the first GEMM (x is [T, K]), 1 for the second (x is [n_slots, K]).
+ * Weights carry a leading expert dimension: qweight [E, K, N/8], scales [E, K/G, N],
+ * qzeros [E, K/G, N/8].  y is fp16 [n_slots, N].  Rows of y whose slot was dropped by the
+ * align step are not written.  Stands in for the fused-MoE expert GEMMs (same models). */
+int awqmi_moe_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
+                       const int32_t* qzeros, void* y_f16, const int32_t* sorted_token_ids,
+                       const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                       const float* topk_weights, int n_slots, int a_row_div, int E, int K, int N,
+                       int group, int split_k, void* workspace, size_t workspace_bytes,
+                       void* stream);
+
+/* out[r, i] = silu(in[r, i]) * in[r, inter + i], in fp16 [rows, 2*inter] ([gate | up]),
+ * out fp16 [rows, inter]; fp32 math.  The activation between the two expert GEMMs. */
+int awqmi_silu_and_mul_f16(const void* in_f16, void* out_f16, int rows, int inter, void* stream);
+
+/* out[t, :] = sum over the topk slot rows in[t*topk + j, :], fp32 sum, fp16 out. */
+int awqmi_moe_sum_f16(const void* in_f16, void* out_f16, int T, int topk, int H, void* stream);
+
+/* Development hook: choose among equivalent kernel variants of the skinny GEMM
+ * (-1 = library default).  Returns the previous value.  Not part of the stable surface. */
+int awqmi_set_gemv_variant(int variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AWQ_MI355X_H */

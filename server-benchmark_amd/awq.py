@@ -1,0 +1,180 @@
+"""AWQConfig / AWQLinearMethod / AWQMoEMethod: the layer-level surface a vLLM model executor
+drives for an AWQ checkpoint (the servers the benchmark harness starts at reference
+utils/generate_compose.py:85-93 pick this method from the checkpoint's quantization_config
+because no --quantization flag is passed).  Same method names, argument meaning and registered
+parameter names (`qweight`, `qzeros`, `scales`), so AWQ state dicts load unchanged; the
+layers are plain torch.nn.Module objects and nothing here imports vLLM.
+"""
+from __future__ import annotations
+
+from typing import Any, Optional
+
+import torch
+from torch.nn import Parameter
+
+from . import ops
+
+
+def _first_key(config: dict, keys, default=None, required=True):
+    for k in keys:
+        if k in config:
+            return config[k]
+    if required:
+        raise ValueError(f"none of {list(keys)} found in the quantization config")
+    return default
+
+
+class AWQConfig:
+    """weight_bits must be 4; pack_factor = 32 / weight_bits = 8; group_size -1 means one
+    group spanning all of K."""
+
+    def __init__(self, weight_bits: int, group_size: int, zero_point: bool,
+                 modules_to_not_convert: Optional[list] = None):
+        if weight_bits != 4:
+            raise ValueError(f"AWQ here supports 4-bit weights only, got {weight_bits} bits")
+        self.weight_bits = weight_bits
+        self.group_size = group_size
+        self.zero_point = zero_point
+        self.modules_to_not_convert = list(modules_to_not_convert or [])
+        self.pack_factor = 32 // weight_bits
+
+    def __repr__(self):
+        return (f"AWQConfig(weight_bits={self.weight_bits}, group_size={self.group_size}, "
+                f"zero_point={self.zero_point}, modules_to_not_convert={self.modules_to_not_convert})")
+
+    @staticmethod
+    def get_name() -> str:
+        return "awq"
+
+    @staticmethod
+    def get_supported_act_dtypes():
+        return [torch.float16]
+
+    @staticmethod
+    def get_config_filenames():
+        return ["quant_config.json", "quantize_config.json"]
+
+    @classmethod
+    def from_config(cls, config: dict) -> "AWQConfig":
+        bits = _first_key(config, ("w_bit", "bits"))
+        group = _first_key(config, ("q_group_size", "group_size"))
+        zp = _first_key(config, ("zero_point",))
+        skip = _first_key(config, ("modules_to_not_convert",), default=None, required=False)
+        return cls(int(bits), int(group), bool(zp), skip)
+
+    def is_skipped(self, prefix: str) -> bool:
+        return any(name in prefix for name in self.modules_to_not_convert)
+
+    def get_quant_method(self, layer: torch.nn.Module, prefix: str = ""):
+        """AWQLinearMethod for a linear layer, AWQMoEMethod for a layer flagged as fused MoE
+        (`layer.is_fused_moe`), None for modules listed in modules_to_not_convert."""
+        if self.is_skipped(prefix):
+            return None
+        if getattr(layer, "is_fused_moe", False):
+            return AWQMoEMethod(self)
+        return AWQLinearMethod(self)
+
+
+def _register(layer, name, tensor, attrs: dict[str, Any]):
+    p = Parameter(tensor, requires_grad=False)
+    for k, v in attrs.items():
+        setattr(p, k, v)
+    layer.register_parameter(name, p)
+
+
+class AWQLinearMethod:
+    def __init__(self, quant_config: AWQConfig):
+        self.quant_config = quant_config
+
+    def create_weights(self, layer: torch.nn.Module, input_size_per_partition: int,
+                       output_partition_sizes: list, input_size: int, output_size: int,
+                       params_dtype: torch.dtype, **extra_weight_attrs):
+        cfg = self.quant_config
+        group = cfg.group_size if cfg.group_size != -1 else input_size
+        if input_size_per_partition % group != 0:
+            raise ValueError("The input size is not aligned with the quantized weight shape. "
+                             "This can be caused by too large tensor parallel size.")
+        out_pp = sum(output_partition_sizes)
+        if out_pp % cfg.pack_factor != 0:
+            raise ValueError("The output size is not aligned with the quantized weight shape. "
+                             "This can be caused by too large tensor parallel size.")
+        if params_dtype != torch.float16:
+            raise ValueError("AWQ scales / activations must be float16")
+        dev = extra_weight_attrs.pop("device", None)
+        ngroups = input_size_per_partition // group
+        packed = dict(input_dim=0, output_dim=1, packed_dim=1, pack_factor=cfg.pack_factor)
+        _register(layer, "qweight",
+                  torch.empty(input_size_per_partition, out_pp // cfg.pack_factor, dtype=torch.int32, device=dev),
+                  {**packed, **extra_weight_attrs})
+        _register(layer, "qzeros",
+                  torch.empty(ngroups, out_pp // cfg.pack_factor, dtype=torch.int32, device=dev),
+                  {**packed, **extra_weight_attrs})
+        _register(layer, "scales",
+                  torch.empty(ngroups, out_pp, dtype=params_dtype, device=dev),
+                  {"input_dim": 0, "output_dim": 1, **extra_weight_attrs})
+        layer.input_size_per_partition = input_size_per_partition
+        layer.output_size_per_partition = out_pp
+        layer.output_partition_sizes = list(output_partition_sizes)
+
+    def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
+        for name in ("qweight", "qzeros", "scales"):
+            t = getattr(layer, name)
+            setattr(layer, name, Parameter(t.data.contiguous(), requires_grad=False))
+
+    def apply(self, layer: torch.nn.Module, x: torch.Tensor,
+              bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        qweight, scales, qzeros = layer.qweight, layer.scales, layer.qzeros
+        out_shape = x.shape[:-1] + (qweight.shape[-1] * self.quant_config.pack_factor,)
+        x2 = x.reshape(-1, x.shape[-1])
+        if not x2.is_contiguous():
+            x2 = x2.contiguous()
+        out = ops.awq_gemm(x2, qweight, scales, qzeros, 0)
+        if bias is not None:
+            out.add_(bias)
+        return out.reshape(out_shape)
+
+
+class AWQMoEMethod:
+    """Fused-MoE counterpart: w13 ([gate | up]) and w2 expert stacks in AWQ layout."""
+
+    def __init__(self, quant_config: AWQConfig):
+        self.quant_config = quant_config
+
+    def create_weights(self, layer: torch.nn.Module, num_experts: int, hidden_size: int,
+                       intermediate_size_per_partition: int, params_dtype: torch.dtype,
+                       **extra_weight_attrs):
+        cfg = self.quant_config
+        pf = cfg.pack_factor
+        dev = extra_weight_attrs.pop("device", None)
+        I = intermediate_size_per_partition
+
+        def grp(k):
+            g = cfg.group_size if cfg.group_size != -1 else k
+            if k % g != 0:
+                raise ValueError(f"K={k} is not a multiple of the group size {g}")
+            return k // g
+
+        shapes = {
+            "w13_qweight": ((num_experts, hidden_size, 2 * I // pf), torch.int32),
+            "w13_scales": ((num_experts, grp(hidden_size), 2 * I), params_dtype),
+            "w13_qzeros": ((num_experts, grp(hidden_size), 2 * I // pf), torch.int32),
+            "w2_qweight": ((num_experts, I, hidden_size // pf), torch.int32),
+            "w2_scales": ((num_experts, grp(I), hidden_size), params_dtype),
+            "w2_qzeros": ((num_experts, grp(I), hidden_size // pf), torch.int32),
+        }
+        for name, (shape, dt) in shapes.items():
+            _register(layer, name, torch.empty(shape, dtype=dt, device=dev), dict(extra_weight_attrs))
+
+    def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
+        for name in ("w13_qweight", "w13_scales", "w13_qzeros", "w2_qweight", "w2_scales", "w2_qzeros"):
+            t = getattr(layer, name)
+            setattr(layer, name, Parameter(t.data.contiguous(), requires_grad=False))
+
+    def apply(self, layer: torch.nn.Module, x: torch.Tensor, router_logits: torch.Tensor, top_k: int,
+              renormalize: bool = True) -> torch.Tensor:
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1]).contiguous()
+        out = ops.fused_moe_awq(x2, (layer.w13_qweight, layer.w13_scales, layer.w13_qzeros),
+                                (layer.w2_qweight, layer.w2_scales, layer.w2_qzeros),
+                                router_logits.reshape(-1, router_logits.shape[-1]), top_k, renormalize)
+        return out.reshape(shape)

@@ -1,0 +1,345 @@
+// C ABI of libawq_mi355x.so: host-side validation and launch of the gfx950 kernels.
+// Every entry point checks its arguments before touching the device, launches on the
+// caller's stream and returns; nothing here allocates, synchronises or keeps state apart
+// from the thread-local last HIP error and the development variant switch.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <type_traits>
+
+#include "../../include/awq_mi355x.h"
+#include "awq_dequant.hpp"
+#include "awq_gemm_mfma.hpp"
+#include "awq_gemv.hpp"
+#include "awq_moe.hpp"
+
+using namespace awqmi;
+
+namespace {
+
+thread_local int t_last_hip_error = 0;
+std::atomic<int> g_gemv_variant{-1};
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int launch_status() {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    t_last_hip_error = (int)e;
+    return AWQMI_LAUNCH_FAILED;
+  }
+  return AWQMI_OK;
+}
+
+inline int norm_group(int K, int group) { return group <= 0 ? K : group; }
+
+int check_awq_shape(int K, int N, int G) {
+  if (K <= 0 || N <= 0 || G <= 0) return AWQMI_BAD_SHAPE;
+  if (N % 8 != 0 || K % G != 0) return AWQMI_BAD_SHAPE;
+  return AWQMI_OK;
+}
+
+// tiled skinny kernel covers: K % 128 == 0 and G in {32, 64, 128 * i}
+inline bool gemv_tiled_ok(int K, int G) {
+  return K % 128 == 0 && (G == 32 || G == 64 || G % 128 == 0);
+}
+inline int gemv_gmode(int G) { return G == 32 ? 0 : (G == 64 ? 1 : (G == 128 ? 2 : 3)); }
+
+inline int gemv_wpl(int N) {
+  const int v = g_gemv_variant.load(std::memory_order_relaxed);
+  const bool want1 = v >= 0 && (v & 1);
+  return (want1 || (N / 8) % 2 != 0) ? 1 : 2;
+}
+
+// Cost model for split-K: bytes moved (weights + fp32 partials out and back) divided by the
+// fraction of the chip's wave slots the launch fills.
+int pick_split_k(int rows, int K, int N, int G, long long blocks_z) {
+  const int nchunks = K / 128;
+  const int ncb = (N + 255) / 256;
+  const double wbytes = (double)K * N / 2.0 * (double)blocks_z;
+  int best = 1;
+  double best_cost = 1e300;
+  const int max_split = nchunks < AWQMI_MAX_SPLIT_K ? nchunks : AWQMI_MAX_SPLIT_K;
+  for (int s = 1; s <= max_split; ++s) {
+    const double waves = (double)ncb * blocks_z * 4.0 * s;
+    const double fill = waves >= 2048.0 ? 1.0 : waves / 2048.0;
+    const double pbytes = s > 1 ? 2.0 * s * rows * (double)N * 4.0 * blocks_z : 0.0;
+    // a wave with under one chunk of work is pure overhead
+    const double idle = (4.0 * s > nchunks) ? (4.0 * s) / nchunks : 1.0;
+    const double cost = (wbytes + pbytes) / fill * idle;
+    if (cost < best_cost * 0.999) { best_cost = cost; best = s; }
+  }
+  (void)G;
+  return best;
+}
+
+inline size_t gemv_partial_bytes(int N, int split, long long blocks_z) {
+  if (split <= 1) return 0;
+  const size_t npad = ((size_t)N + 255) / 256 * 256;
+  return (size_t)split * (size_t)blocks_z * 16 * npad * sizeof(float);
+}
+
+template <int WPL, bool MOE>
+void launch_gemv(const GemvParams& p, int gmode, dim3 grid, hipStream_t st) {
+  switch (gmode) {
+    case 0: hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MOE>), grid, dim3(256), 0, st, p); break;
+    case 1: hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MOE>), grid, dim3(256), 0, st, p); break;
+    case 2: hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MOE>), grid, dim3(256), 0, st, p); break;
+    default: hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MOE>), grid, dim3(256), 0, st, p); break;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int awqmi_version(void) { return AWQMI_VERSION; }
+
+const char* awqmi_status_string(int s) {
+  switch (s) {
+    case AWQMI_OK: return "ok";
+    case AWQMI_BAD_SHAPE: return "bad shape (need N % 8 == 0, K % group == 0, positive sizes)";
+    case AWQMI_BAD_ALIGN: return "pointer not 16-byte aligned";
+    case AWQMI_WORKSPACE_TOO_SMALL: return "workspace too small";
+    case AWQMI_UNSUPPORTED_GROUP: return "unsupported group size";
+    case AWQMI_LAUNCH_FAILED: return "kernel launch failed";
+    case AWQMI_NULL_POINTER: return "null pointer";
+    case AWQMI_BAD_ARGUMENT: return "bad argument";
+    default: return "unknown status";
+  }
+}
+
+int awqmi_last_hip_error(void) { return t_last_hip_error; }
+
+int awqmi_set_gemv_variant(int v) { return g_gemv_variant.exchange(v); }
+
+int awqmi_dequantize_f16(const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                         void* out, int K, int N, int group, void* stream) {
+  if (!qweight || !scales || !qzeros || !out) return AWQMI_NULL_POINTER;
+  const int G = norm_group(K, group);
+  if (int st = check_awq_shape(K, N, G)) return st;
+  if (!aligned16(scales) || !aligned16(out) || !aligned16(qweight) || !aligned16(qzeros))
+    return AWQMI_BAD_ALIGN;
+  const int NW = N / 8;
+  hipStream_t st = (hipStream_t)stream;
+  const uint32_t* qw = reinterpret_cast<const uint32_t*>(qweight);
+  const uint32_t* qz = reinterpret_cast<const uint32_t*>(qzeros);
+  const half_t* sc = reinterpret_cast<const half_t*>(scales);
+  half_t* o = reinterpret_cast<half_t*>(out);
+  const unsigned gx = (NW + 255) / 256;
+#define AWQMI_DQ(R)                                                                              \
+  hipLaunchKernelGGL((awq_dequant_kernel<R>), dim3(gx, K / R), dim3(256), 0, st, qw, sc, qz, o, K, \
+                     NW, G)
+  if (G % 16 == 0) AWQMI_DQ(16);
+  else if (G % 8 == 0) AWQMI_DQ(8);
+  else if (G % 4 == 0) AWQMI_DQ(4);
+  else if (G % 2 == 0) AWQMI_DQ(2);
+  else AWQMI_DQ(1);
+#undef AWQMI_DQ
+  return launch_status();
+}
+
+int awqmi_gemm_auto_split_k(int M, int K, int N, int group) {
+  const int G = norm_group(K, group);
+  if (check_awq_shape(K, N, G) != AWQMI_OK || M <= 0) return 1;
+  if (M > 16 || !gemv_tiled_ok(K, G)) return 1;
+  return pick_split_k(M, K, N, G, 1);
+}
+
+size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
+  if (M <= 0 || K <= 0 || N <= 0) return 0;
+  if (M > 16) return AWQMI_WS_COUNTER_BYTES;
+  int s = split_k;
+  if (s <= 0) s = (K % 128 == 0) ? pick_split_k(M, K, N, 128, 1) : 1;
+  return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, s, 1);
+}
+
+int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                   void* y, void* workspace, size_t workspace_bytes, int M, int K, int N, int group,
+                   int split_k, void* stream) {
+  if (!x || !qweight || !scales || !qzeros || !y) return AWQMI_NULL_POINTER;
+  const int G = norm_group(K, group);
+  if (int st = check_awq_shape(K, N, G)) return st;
+  if (M <= 0) return AWQMI_BAD_SHAPE;
+  if (split_k < 0 || split_k > AWQMI_MAX_SPLIT_K) return AWQMI_BAD_ARGUMENT;
+  if (!aligned16(x) || !aligned16(scales) || !aligned16(qweight) || !aligned16(qzeros) ||
+      !aligned16(y))
+    return AWQMI_BAD_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  const int NW = N / 8;
+  const uint32_t* qw = reinterpret_cast<const uint32_t*>(qweight);
+  const uint32_t* qz = reinterpret_cast<const uint32_t*>(qzeros);
+  const half_t* sc = reinterpret_cast<const half_t*>(scales);
+  const half_t* xx = reinterpret_cast<const half_t*>(x);
+  half_t* yy = reinterpret_cast<half_t*>(y);
+
+  if (M <= 16 && gemv_tiled_ok(K, G)) {
+    int split = split_k > 0 ? split_k : pick_split_k(M, K, N, G, 1);
+    const int nchunks = K / 128;
+    if (split > nchunks) split = nchunks;
+    const int wpl = gemv_wpl(N);
+    const int ncb = (NW + 16 * wpl - 1) / (16 * wpl);
+    if (split > 1) {
+      if (!workspace) return AWQMI_NULL_POINTER;
+      if (!aligned16(workspace)) return AWQMI_BAD_ALIGN;
+      if ((size_t)ncb * sizeof(int) > AWQMI_WS_COUNTER_BYTES) return AWQMI_BAD_SHAPE;
+      if (workspace_bytes < AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, split, 1))
+        return AWQMI_WORKSPACE_TOO_SMALL;
+    }
+    GemvParams p{};
+    p.x = xx; p.qw = qw; p.sc = sc; p.qz = qz; p.y = yy;
+    p.cnt = reinterpret_cast<int*>(workspace);
+    p.part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
+                       : nullptr;
+    p.M = M; p.K = K; p.N = N; p.NW = NW; p.G = G;
+    p.nchunks = nchunks; p.cpg = G >= 128 ? G / 128 : 1; p.split_k = split; p.ncb = ncb;
+    const dim3 grid(ncb, split, 1);
+    if (wpl == 2) launch_gemv<2, false>(p, gemv_gmode(G), grid, st);
+    else launch_gemv<1, false>(p, gemv_gmode(G), grid, st);
+    return launch_status();
+  }
+
+  if (M > 16 && K % PF_BK == 0 && G % 8 == 0) {
+    static std::atomic<bool> attr_set{false};
+    if (!attr_set.load(std::memory_order_acquire)) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(awq_gemm_mfma_kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               PF_LDS_BYTES);
+      if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
+      attr_set.store(true, std::memory_order_release);
+    }
+    MfmaGemmParams p{};
+    p.x = xx; p.qw = qw; p.sc = sc; p.qz = qz; p.y = yy;
+    p.M = M; p.K = K; p.N = N; p.NW = NW; p.G = G;
+    p.mt = (M + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
+    p.total = p.mt * p.nt; p.per_xcd = (p.total + 7) / 8;
+    hipLaunchKernelGGL(awq_gemm_mfma_kernel, dim3(p.per_xcd * 8), dim3(256), PF_LDS_BYTES, st, p);
+    return launch_status();
+  }
+
+  hipLaunchKernelGGL(awq_gemm_generic_kernel, dim3((NW + 255) / 256, M), dim3(256), 0, st, xx, qw, sc,
+                     qz, yy, M, K, NW, G);
+  return launch_status();
+}
+
+int awqmi_moe_topk_softmax_f32(const float* logits, int T, int E, int topk, int renormalize,
+                               int32_t* topk_ids, float* topk_weights, void* stream) {
+  if (!logits || !topk_ids || !topk_weights) return AWQMI_NULL_POINTER;
+  if (T <= 0 || E <= 0) return AWQMI_BAD_SHAPE;
+  if (E > AWQMI_MAX_EXPERTS || topk <= 0 || topk > E || topk > 64) return AWQMI_BAD_ARGUMENT;
+  hipLaunchKernelGGL(moe_topk_softmax_kernel, dim3((T + 3) / 4), dim3(256), 0, (hipStream_t)stream,
+                     logits, T, E, topk, renormalize, topk_ids, topk_weights);
+  return launch_status();
+}
+
+size_t awqmi_moe_align_capacity(int n_slots, int E, int tile_m) {
+  if (n_slots < 0 || E <= 0 || tile_m <= 0) return 0;
+  const size_t worst = (size_t)n_slots + (size_t)E * (tile_m - 1);
+  return (worst + tile_m - 1) / tile_m * tile_m;
+}
+
+int awqmi_moe_align(const int32_t* topk_ids, int n_slots, int E, int tile_m, int32_t* sorted_token_ids,
+                    int32_t* expert_ids, int32_t* num_tokens_post_padded, void* stream) {
+  if (!topk_ids || !sorted_token_ids || !expert_ids || !num_tokens_post_padded)
+    return AWQMI_NULL_POINTER;
+  if (n_slots <= 0 || E <= 0) return AWQMI_BAD_SHAPE;
+  if (E > AWQMI_MAX_EXPERTS || tile_m <= 0 || tile_m > 4096) return AWQMI_BAD_ARGUMENT;
+  const int cap = (int)awqmi_moe_align_capacity(n_slots, E, tile_m);
+  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(512), (size_t)10 * E * sizeof(int),
+                     (hipStream_t)stream, topk_ids, n_slots, E, tile_m, cap, sorted_token_ids,
+                     expert_ids, num_tokens_post_padded);
+  return launch_status();
+}
+
+static int moe_pick_split(int n_slots, int E, int K, int N, int G, int nblk, int ncb) {
+  // blocks that will actually run: at most one per 16 slots plus one per expert touched
+  long long live = (n_slots + 15) / 16;
+  const long long touched = n_slots < E ? n_slots : E;
+  if (live < touched) live = touched;
+  int s = pick_split_k(16, K, N, G, live);
+  if ((size_t)nblk * ncb * sizeof(int) > AWQMI_WS_COUNTER_BYTES) s = 1;
+  return s;
+}
+
+size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int split_k) {
+  if (n_slots <= 0 || E <= 0 || K <= 0 || N <= 0) return 0;
+  const int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, AWQMI_MOE_TILE_M) / AWQMI_MOE_TILE_M);
+  int s = split_k;
+  if (s <= 0) s = (K % 128 == 0) ? moe_pick_split(n_slots, E, K, N, 128, nblk, (N + 127) / 128) : 1;
+  return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, s, nblk);
+}
+
+int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                       void* y, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                       const int32_t* num_tokens_post_padded, const float* topk_weights, int n_slots,
+                       int a_row_div, int E, int K, int N, int group, int split_k, void* workspace,
+                       size_t workspace_bytes, void* stream) {
+  if (!x || !qweight || !scales || !qzeros || !y || !sorted_token_ids || !expert_ids ||
+      !num_tokens_post_padded)
+    return AWQMI_NULL_POINTER;
+  const int G = norm_group(K, group);
+  if (int st = check_awq_shape(K, N, G)) return st;
+  if (n_slots <= 0 || E <= 0) return AWQMI_BAD_SHAPE;
+  if (a_row_div <= 0 || split_k < 0 || split_k > AWQMI_MAX_SPLIT_K || E > AWQMI_MAX_EXPERTS)
+    return AWQMI_BAD_ARGUMENT;
+  if (!gemv_tiled_ok(K, G)) return AWQMI_UNSUPPORTED_GROUP;
+  if (!aligned16(x) || !aligned16(scales) || !aligned16(qweight) || !aligned16(qzeros) ||
+      !aligned16(y))
+    return AWQMI_BAD_ALIGN;
+  const int NW = N / 8;
+  const int wpl = gemv_wpl(N);
+  const int ncb = (NW + 16 * wpl - 1) / (16 * wpl);
+  const int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, AWQMI_MOE_TILE_M) / AWQMI_MOE_TILE_M);
+  int split = split_k > 0 ? split_k : moe_pick_split(n_slots, E, K, N, G, nblk, ncb);
+  const int nchunks = K / 128;
+  if (split > nchunks) split = nchunks;
+  if (split > 1) {
+    if (!workspace) return AWQMI_NULL_POINTER;
+    if (!aligned16(workspace)) return AWQMI_BAD_ALIGN;
+    if ((size_t)nblk * ncb * sizeof(int) > AWQMI_WS_COUNTER_BYTES) return AWQMI_BAD_ARGUMENT;
+    if (workspace_bytes < AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, split, nblk))
+      return AWQMI_WORKSPACE_TOO_SMALL;
+  }
+  GemvParams p{};
+  p.x = reinterpret_cast<const half_t*>(x);
+  p.qw = reinterpret_cast<const uint32_t*>(qweight);
+  p.sc = reinterpret_cast<const half_t*>(scales);
+  p.qz = reinterpret_cast<const uint32_t*>(qzeros);
+  p.y = reinterpret_cast<half_t*>(y);
+  p.cnt = reinterpret_cast<int*>(workspace);
+  p.part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
+                     : nullptr;
+  p.M = 16; p.K = K; p.N = N; p.NW = NW; p.G = G;
+  p.nchunks = nchunks; p.cpg = G >= 128 ? G / 128 : 1; p.split_k = split; p.ncb = ncb;
+  p.sorted_ids = sorted_token_ids; p.expert_ids = expert_ids; p.n_post_pad = num_tokens_post_padded;
+  p.topk_w = topk_weights; p.n_slots = n_slots; p.a_row_div = a_row_div;
+  p.w_stride = (long long)K * NW; p.s_stride = (long long)(K / G) * N; p.z_stride = (long long)(K / G) * NW;
+  const dim3 grid(ncb, split, nblk);
+  if (wpl == 2) launch_gemv<2, true>(p, gemv_gmode(G), grid, (hipStream_t)stream);
+  else launch_gemv<1, true>(p, gemv_gmode(G), grid, (hipStream_t)stream);
+  return launch_status();
+}
+
+int awqmi_silu_and_mul_f16(const void* in, void* out, int rows, int inter, void* stream) {
+  if (!in || !out) return AWQMI_NULL_POINTER;
+  if (rows <= 0 || inter <= 0 || inter % 8 != 0) return AWQMI_BAD_SHAPE;
+  if (!aligned16(in) || !aligned16(out)) return AWQMI_BAD_ALIGN;
+  const size_t n = (size_t)rows * (inter / 8);
+  hipLaunchKernelGGL(silu_and_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, reinterpret_cast<const half_t*>(in),
+                     reinterpret_cast<half_t*>(out), rows, inter);
+  return launch_status();
+}
+
+int awqmi_moe_sum_f16(const void* in, void* out, int T, int topk, int H, void* stream) {
+  if (!in || !out) return AWQMI_NULL_POINTER;
+  if (T <= 0 || topk <= 0 || H <= 0 || H % 8 != 0) return AWQMI_BAD_SHAPE;
+  if (!aligned16(in) || !aligned16(out)) return AWQMI_BAD_ALIGN;
+  const size_t n = (size_t)T * (H / 8);
+  hipLaunchKernelGGL(moe_sum_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, reinterpret_cast<const half_t*>(in),
+                     reinterpret_cast<half_t*>(out), T, topk, H);
+  return launch_status();
+}
+
+}  // extern "C"

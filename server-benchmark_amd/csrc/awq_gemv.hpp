@@ -1,0 +1,316 @@
+// Skinny AWQ GEMM (M <= 16 rows per launch block): Y[M,N] = X[M,K] @ dequant(W), HBM-bound.
+//
+// One wave owns a block of 128*WPL output columns and a contiguous range of 128-row chunks
+// of K.  Per 32-row step each lane loads 8 rows x WPL packed words (16 lanes side by side
+// cover 64*WPL contiguous bytes of a row, the four 16-lane groups take four 8-row slabs),
+// turns the 8x8 nibble block of every word into the B operand of v_mfma_f32_16x16x32_f16
+// with one v_perm_b32 + two v_and_or_b32 + two v_pk_add_f16 per four weights, and feeds it
+// against the 16xK activation slab (A operand, straight from global memory).  The integer
+// difference (w - z) goes through the matrix core; the group scale is applied to the
+// per-group accumulator in fp32, so no per-weight multiply is spent.  Four waves of a
+// workgroup split the workgroup's K range and meet in LDS; workgroups of a split-K launch
+// meet through fp32 partials in the workspace, summed in fixed order by whichever
+// workgroup arrives last (arrival counter per column block, left at zero).
+#pragma once
+#include "awq_common.hpp"
+
+namespace awqmi {
+
+struct GemvParams {
+  const half_t* x;
+  const uint32_t* qw;
+  const half_t* sc;
+  const uint32_t* qz;
+  half_t* y;
+  float* part;  // [split][nblk*ncb][16][128*WPL] fp32 partial tiles (tile-major columns)
+  int* cnt;     // [nblk*ncb] arrival counters
+  int M, K, N, NW, G;
+  int nchunks;  // K / 128
+  int cpg;      // chunks per group when G >= 128
+  int split_k;
+  int ncb;      // column blocks
+  // expert-grouped launch
+  const int* sorted_ids;
+  const int* expert_ids;
+  const int* n_post_pad;
+  const float* topk_w;
+  int n_slots;
+  int a_row_div;
+  long long w_stride, s_stride, z_stride;  // elements per expert
+};
+
+template <int WPL>
+struct WordVec;
+template <>
+struct WordVec<1> {
+  typedef uint32_t type;
+  static __device__ __forceinline__ uint32_t get(uint32_t v, int) { return v; }
+};
+template <>
+struct WordVec<2> {
+  typedef u2v type;
+  static __device__ __forceinline__ uint32_t get(u2v v, int w) { return w ? v.y : v.x; }
+};
+
+// GMODE: 0 -> G = 32, 1 -> G = 64, 2 -> G = 128, 3 -> G = 128 * cpg (cpg > 1)
+template <int WPL, int GMODE, bool MOE>
+struct GemvWave {
+  static constexpr int NT = 8 * WPL;                                    // 16-col tiles / wave
+  static constexpr int KSPG = GMODE == 0 ? 1 : (GMODE == 1 ? 2 : 4);   // 32-row steps / group
+  typedef typename WordVec<WPL>::type qvec;
+
+  const GemvParams& p;
+  const uint32_t* qw;  // lane's column already applied
+  const half_t* sc;
+  const uint32_t* qz;
+  const half_t* xrow;  // lane's activation row, 8h applied
+  int h;
+
+  qvec q[4][8];
+  u4v a[4];
+  f4 acc[NT];
+  f4 accg[NT];
+  qvec zcur, znext;
+  u4v scur[WPL], snext[WPL];
+  uint32_t zlo[WPL][4], zhi[WPL][4];  // (1024+z, 1024+z) / (64+z, 64+z) per byte of the word
+
+  __device__ __forceinline__ GemvWave(const GemvParams& pp) : p(pp) {}
+
+  __device__ __forceinline__ void issue(int s, int c) {
+    const size_t row0 = (size_t)c * 128 + 32 * s + 8 * h;
+    const qvec* src = reinterpret_cast<const qvec*>(qw + row0 * p.NW);
+    const size_t stride = (size_t)p.NW / WPL;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) q[s][i] = __builtin_nontemporal_load(src + i * stride);
+    a[s] = *reinterpret_cast<const u4v*>(xrow + (size_t)c * 128 + 32 * s);
+  }
+
+  __device__ __forceinline__ void load_group(int g, qvec& z, u4v (&s)[WPL]) {
+    z = *reinterpret_cast<const qvec*>(qz + (size_t)g * p.NW);
+#pragma unroll
+    for (int w = 0; w < WPL; ++w) s[w] = *reinterpret_cast<const u4v*>(sc + (size_t)g * p.N + 8 * w);
+  }
+
+  __device__ __forceinline__ void build_zdup() {
+#pragma unroll
+    for (int w = 0; w < WPL; ++w) {
+      const uint32_t zw = WordVec<WPL>::get(zcur, w);
+      uint32_t t;
+      t = byte_pair<0>(zw, zw); zlo[w][0] = (t & MASK_LO) | MAGIC_LO; zhi[w][0] = (t & MASK_HI) | MAGIC_HI;
+      t = byte_pair<1>(zw, zw); zlo[w][1] = (t & MASK_LO) | MAGIC_LO; zhi[w][1] = (t & MASK_HI) | MAGIC_HI;
+      t = byte_pair<2>(zw, zw); zlo[w][2] = (t & MASK_LO) | MAGIC_LO; zhi[w][2] = (t & MASK_HI) | MAGIC_HI;
+      t = byte_pair<3>(zw, zw); zlo[w][3] = (t & MASK_LO) | MAGIC_LO; zhi[w][3] = (t & MASK_HI) | MAGIC_HI;
+    }
+  }
+
+  template <int B>
+  __device__ __forceinline__ void tile_pair(int s, int w, bool first) {
+    u4v lo, hi;
+#pragma unroll
+    for (int rp = 0; rp < 4; ++rp) {
+      const uint32_t t = byte_pair<B>(WordVec<WPL>::get(q[s][2 * rp + 1], w),
+                                      WordVec<WPL>::get(q[s][2 * rp], w));
+      lo[rp] = (t & MASK_LO) | MAGIC_LO;
+      hi[rp] = (t & MASK_HI) | MAGIC_HI;
+    }
+    const uint32_t zl = zlo[w][B], zh = zhi[w][B];
+    const h8 blo = as_h8(lo) - as_h8(u4v{zl, zl, zl, zl});
+    const h8 bhi = as_h8(hi) - as_h8(u4v{zh, zh, zh, zh});
+    const h8 av = as_h8(a[s]);
+    const int t0 = w * 8 + 2 * B;
+    const f4 zero = {0.f, 0.f, 0.f, 0.f};
+    accg[t0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, blo, first ? zero : accg[t0], 0, 0, 0);
+    accg[t0 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bhi, first ? zero : accg[t0 + 1], 0, 0, 0);
+  }
+
+  __device__ __forceinline__ void compute(int s, bool first) {
+#pragma unroll
+    for (int w = 0; w < WPL; ++w) {
+      tile_pair<0>(s, w, first);
+      tile_pair<1>(s, w, first);
+      tile_pair<2>(s, w, first);
+      tile_pair<3>(s, w, first);
+    }
+  }
+
+  __device__ __forceinline__ void flush() {
+#pragma unroll
+    for (int w = 0; w < WPL; ++w) {
+      const h8 sv = as_h8(scur[w]);
+#pragma unroll
+      for (int nib = 0; nib < 8; ++nib) {
+        const float s = (float)sv[awq_col_of_nibble(nib)];
+        const int t = w * 8 + nib;
+        acc[t] += s * accg[t];
+      }
+    }
+  }
+
+  // one 128-row chunk; REFILL: chunk c+1 belongs to this wave too
+  template <bool REFILL>
+  __device__ __forceinline__ void chunk(int c, int c_begin, int c_end) {
+    if (GMODE == 2) {
+      build_zdup();
+      if (REFILL) load_group(c + 1, znext, snext);
+    } else if (GMODE == 3) {
+      if (c == c_begin || c % p.cpg == 0) {
+        load_group(c / p.cpg, zcur, scur);
+        build_zdup();
+#pragma unroll
+        for (int t = 0; t < NT; ++t) accg[t] = f4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      if (GMODE < 2 && s % KSPG == 0) {
+        load_group((c * 4 + s) / KSPG, zcur, scur);
+        build_zdup();
+      }
+      compute(s, GMODE == 3 ? false : (s % KSPG == 0));
+      if (REFILL) issue(s, c + 1);
+      if (GMODE < 2 && (s + 1) % KSPG == 0) flush();
+    }
+    if (GMODE == 2) {
+      flush();
+      if (REFILL) {
+        zcur = znext;
+#pragma unroll
+        for (int w = 0; w < WPL; ++w) scur[w] = snext[w];
+      }
+    } else if (GMODE == 3) {
+      if (c + 1 == c_end || (c + 1) % p.cpg == 0) flush();
+    }
+  }
+
+  __device__ __forceinline__ void run(int c_begin, int c_end) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
+    if (c_begin >= c_end) return;
+    if (GMODE == 2) load_group(c_begin, zcur, scur);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) issue(s, c_begin);
+    int c = c_begin;
+    for (; c + 1 < c_end; ++c) chunk<true>(c, c_begin, c_end);
+    chunk<false>(c, c_begin, c_end);
+  }
+};
+
+template <int WPL, int GMODE, bool MOE>
+__global__ __launch_bounds__(256, WPL == 1 ? 2 : 1) void awq_gemv_kernel(const GemvParams p) {
+  constexpr int NT = 8 * WPL;
+  constexpr int CB = 128 * WPL;
+  constexpr int RS = NT * 16 + 4;  // LDS row stride in floats: 4h rows land 16 banks apart
+  __shared__ float red[2][16][RS];
+  __shared__ int s_last;
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, h = lane >> 4;
+  const int cb = blockIdx.x, sp = blockIdx.y;
+  int blk = 0;
+  const uint32_t* qw = p.qw;
+  const half_t* sc = p.sc;
+  const uint32_t* qz = p.qz;
+  if (MOE) {
+    blk = blockIdx.z;
+    if (blk * 16 >= *p.n_post_pad) return;
+    const int e = p.expert_ids[blk];
+    qw += (size_t)e * p.w_stride;
+    sc += (size_t)e * p.s_stride;
+    qz += (size_t)e * p.z_stride;
+  }
+
+  // Lanes past the last word column / past the last row read valid memory of column block 0
+  // / row 0 instead; their B column (resp. A row) only feeds outputs that are never stored.
+  int wc = cb * (16 * WPL) + WPL * j;
+  if (wc >= p.NW) wc = 0;
+  size_t arow;
+  if (!MOE) {
+    arow = j < p.M ? (size_t)j : 0;
+  } else {
+    const int sid = p.sorted_ids[blk * 16 + j];
+    arow = sid < p.n_slots ? (size_t)(sid / p.a_row_div) : 0;
+  }
+
+  GemvWave<WPL, GMODE, MOE> w(p);
+  w.qw = qw + wc;
+  w.sc = sc + 8 * (size_t)wc;
+  w.qz = qz + wc;
+  w.xrow = p.x + arow * p.K + 8 * h;
+  w.h = h;
+
+  const long long parts = 4LL * p.split_k;
+  const long long pw = (long long)sp * 4 + wave;
+  const int c_begin = (int)(pw * p.nchunks / parts);
+  const int c_end = (int)((pw + 1) * p.nchunks / parts);
+  w.run(c_begin, c_end);
+
+  // ---- cross-wave sum in LDS: red[b][row][tile*16 + j] ----
+  if (wave >= 2) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave - 2][4 * h + r][t * 16 + j] = w.acc[t][r];
+  }
+  __syncthreads();
+  if (wave < 2) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][4 * h + r][t * 16 + j] += w.acc[t][r];
+  }
+  __syncthreads();
+
+  int rows = p.M;
+  if (MOE) {  // valid slots sit at the front of a block, pads behind them
+    rows = 0;
+    for (int m = 0; m < 16; ++m) rows += p.sorted_ids[blk * 16 + m] < p.n_slots ? 1 : 0;
+  }
+  const int nelem = rows * (NT * 16);
+  if (p.split_k > 1) {
+    // fp32 partial tile of this workgroup, then the arrival counter
+    const size_t tile = (size_t)blk * p.ncb + cb;
+    const size_t ntiles = (size_t)(MOE ? gridDim.z : 1) * p.ncb;
+    float* mine = p.part + ((size_t)sp * ntiles + tile) * (16 * NT * 16);
+    for (int i = tid; i < nelem; i += 256) {
+      const int m = i / (NT * 16), c = i % (NT * 16);
+      mine[i] = red[0][m][c] + red[1][m][c];
+    }
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) s_last = (atomicAdd(p.cnt + tile, 1) == p.split_k - 1);
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    for (int i = tid; i < nelem; i += 256) {
+      float v = 0.f;
+      for (int s = 0; s < p.split_k; ++s)
+        v += __builtin_nontemporal_load(p.part + ((size_t)s * ntiles + tile) * (16 * NT * 16) + i);
+      red[0][i / (NT * 16)][i % (NT * 16)] = v;
+    }
+    if (tid == 0) p.cnt[tile] = 0;
+    __syncthreads();
+  }
+
+  // ---- tile-major LDS -> row-major fp16 output ----
+  const bool summed = p.split_k > 1;
+  for (int i = tid; i < rows * CB; i += 256) {
+    const int m = i / CB, cl = i % CB;
+    const int wl = cl >> 3;                 // word within the block
+    const int jj = wl / WPL, ww = wl % WPL;
+    const int t = ww * 8 + awq_nibble_of_col(cl & 7);
+    const int col = cb * CB + cl;
+    float v = red[0][m][t * 16 + jj];
+    if (!summed) v += red[1][m][t * 16 + jj];
+    if (col >= p.N) continue;
+    if (!MOE) {
+      p.y[(size_t)m * p.N + col] = (half_t)v;
+    } else {
+      const int sid = p.sorted_ids[blk * 16 + m];
+      if (sid < p.n_slots) {
+        if (p.topk_w) v *= p.topk_w[sid];
+        p.y[(size_t)sid * p.N + col] = (half_t)v;
+      }
+    }
+  }
+}
+
+}  // namespace awqmi

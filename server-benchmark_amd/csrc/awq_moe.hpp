@@ -1,0 +1,177 @@
+// Routing-side kernels of the expert-grouped AWQ path: softmax + top-k, the stable
+// sort/pad of routed slots by expert, the SiLU(gate) * up activation between the two expert
+// GEMMs, and the final sum over a token's slots.  All are latency-sized integer / elementwise
+// work; the expert GEMMs themselves are the MOE instantiation of the skinny kernel.
+#pragma once
+#include "awq_common.hpp"
+
+namespace awqmi {
+
+// One wave per token.  Selection runs on the raw logits (softmax is monotonic), ties go to
+// the lowest expert id.  E <= 1024.
+__global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __restrict__ logits, int T,
+                                                               int E, int topk, int renorm,
+                                                               int* __restrict__ ids,
+                                                               float* __restrict__ wts) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  constexpr int PER = 16;  // 64 * 16 = 1024 experts at most
+  float v[PER];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int e = lane + 64 * i;
+    v[i] = e < E ? logits[(size_t)t * E + e] : -INFINITY;
+    mx = fmaxf(mx, v[i]);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int e = lane + 64 * i;
+    if (e < E) sum += __expf(v[i] - mx);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+
+  float sel_sum = 0.f;
+  float my_w = 0.f;   // lane j keeps the weight of pick j (topk <= 64)
+  int my_id = 0;
+  for (int it = 0; it < topk; ++it) {
+    float best = -INFINITY;
+    int bidx = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int e = lane + 64 * i;
+      if (e < E && (v[i] > best)) { best = v[i]; bidx = e; }   // ascending e: first max wins
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o);
+      const int oi = __shfl_xor(bidx, o);
+      if (ob > best || (ob == best && oi < bidx)) { best = ob; bidx = oi; }
+    }
+    const float pw = __expf(best - mx) / sum;
+    sel_sum += pw;
+    if (lane == it) { my_w = pw; my_id = bidx; }
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (lane + 64 * i == bidx) v[i] = -INFINITY;
+  }
+  if (lane < topk) {
+    ids[(size_t)t * topk + lane] = my_id;
+    wts[(size_t)t * topk + lane] = renorm ? my_w / sel_sum : my_w;
+  }
+}
+
+// Single workgroup of 8 waves.  Dynamic LDS: cnt[8][E] + padded[E] + start[E].
+// Wave w owns the contiguous slice [w*seg, (w+1)*seg) of the flat slot list, so placing
+// slices in wave order and slots in index order inside a slice gives a stable sort.
+__global__ __launch_bounds__(512) void moe_align_kernel(const int* __restrict__ ids, int n, int E,
+                                                        int tile_m, int cap,
+                                                        int* __restrict__ sorted,
+                                                        int* __restrict__ expert_ids,
+                                                        int* __restrict__ npp) {
+  extern __shared__ int sm[];
+  int* cnt = sm;             // [8][E], later the running write position
+  int* padded = sm + 8 * E;  // [E]
+  int* start = padded + E;   // [E]
+  __shared__ int s_total;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+
+  for (int i = tid; i < 8 * E; i += 512) cnt[i] = 0;
+  __syncthreads();
+
+  const int seg = ((n + 8 * 64 - 1) / (8 * 64)) * 64;
+  const int sb = wave * seg, se = min(n, sb + seg);
+  for (int i = sb + lane; i < se; i += 64) {
+    const int e = ids[i];
+    if (e >= 0 && e < E) atomicAdd(&cnt[wave * E + e], 1);
+  }
+  __syncthreads();
+
+  for (int e = tid; e < E; e += 512) {
+    int tot = 0;
+    for (int w = 0; w < 8; ++w) tot += cnt[w * E + e];
+    padded[e] = (tot + tile_m - 1) / tile_m * tile_m;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int pos = 0;
+    for (int e = 0; e < E; ++e) { start[e] = pos; pos += padded[e]; }
+    s_total = pos;
+    npp[0] = pos;
+  }
+  __syncthreads();
+  const int total = s_total;
+  for (int e = tid; e < E; e += 512) {
+    int pos = start[e];
+    const int s0 = pos;
+    for (int w = 0; w < 8; ++w) { const int c = cnt[w * E + e]; cnt[w * E + e] = pos; pos += c; }
+    for (int i = pos; i < s0 + padded[e]; ++i) sorted[i] = n;            // pad entries
+    for (int b = 0; b < padded[e] / tile_m; ++b) expert_ids[s0 / tile_m + b] = e;
+  }
+  for (int i = total + tid; i < cap; i += 512) sorted[i] = n;           // unused tail
+  for (int i = total / tile_m + tid; i < cap / tile_m; i += 512) expert_ids[i] = -1;
+  __syncthreads();
+
+  for (int i0 = sb; i0 < se; i0 += 64) {
+    const int i = i0 + lane;
+    int e = i < se ? ids[i] : -1;
+    const bool valid = e >= 0 && e < E;
+    unsigned long long remaining = __ballot(valid);
+    while (remaining) {
+      const int leader = __ffsll((long long)remaining) - 1;
+      const int e0 = __shfl(e, leader);
+      const bool mine = valid && e == e0;
+      const unsigned long long mask = __ballot(mine);
+      const int rank = __popcll(mask & ((1ull << lane) - 1ull));
+      const int base = cnt[wave * E + e0];
+      if (mine) sorted[base + rank] = i;
+      if (lane == leader) cnt[wave * E + e0] = base + __popcll(mask);
+      remaining &= ~mask;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void silu_and_mul_kernel(const half_t* __restrict__ in,
+                                                           half_t* __restrict__ out, int rows,
+                                                           int inter) {
+  // 8 halves per thread; inter % 8 == 0
+  const int per_row = inter / 8;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)rows * per_row) return;
+  const size_t r = idx / per_row, c = (idx % per_row) * 8;
+  const h8 g = *reinterpret_cast<const h8*>(in + r * 2 * inter + c);
+  const h8 u = *reinterpret_cast<const h8*>(in + r * 2 * inter + inter + c);
+  h8 o;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float gv = (float)g[i];
+    o[i] = (half_t)(gv / (1.f + __expf(-gv)) * (float)u[i]);
+  }
+  *reinterpret_cast<h8*>(out + r * inter + c) = o;
+}
+
+__global__ __launch_bounds__(256) void moe_sum_kernel(const half_t* __restrict__ in,
+                                                      half_t* __restrict__ out, int T, int topk,
+                                                      int H) {
+  const int per_row = H / 8;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)T * per_row) return;
+  const size_t t = idx / per_row, c = (idx % per_row) * 8;
+  float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < topk; ++j) {
+    const h8 v = *reinterpret_cast<const h8*>(in + (t * topk + j) * H + c);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s[i] += (float)v[i];
+  }
+  h8 o;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = (half_t)s[i];
+  *reinterpret_cast<h8*>(out + t * H + c) = o;
+}
+
+}  // namespace awqmi

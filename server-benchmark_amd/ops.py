@@ -1,0 +1,226 @@
+"""Operator surface of the AWQ W4A16 path, keeping vLLM's names and argument order:
+
+    awq_dequantize(qweight, scales, zeros, split_k_iters, thx, thy) -> fp16 [K, N]
+    awq_gemm(input, qweight, scales, qzeros, split_k_iters)          -> fp16 [M, N]
+
+plus the fused-MoE pieces (topk_softmax, moe_align_block_size, moe_awq_gemm, silu_and_mul,
+moe_sum).  Each function checks dtype / device / contiguity / shape relations, then calls
+the C ABI with raw device pointers on torch's current stream.  Tensors are torch tensors on a
+ROCm device; torch is used for memory and streams only.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+MOE_TILE_M = 16
+_WS_COUNTER_BYTES = 65536
+_workspaces: dict = {}
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _need(t: torch.Tensor, name: str, dtype, ndim=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if ndim is not None and t.dim() != ndim:
+        raise ValueError(f"{name} must have {ndim} dims, got shape {tuple(t.shape)}")
+
+
+def _awq_shapes(qweight, scales, qzeros, lead=0):
+    K, NW = qweight.shape[lead], qweight.shape[lead + 1]
+    N = NW * 8
+    groups = scales.shape[lead]
+    if groups <= 0 or K % groups != 0:
+        raise ValueError(f"scales rows {groups} must divide K={K}")
+    if tuple(scales.shape[lead:]) != (groups, N):
+        raise ValueError(f"scales shape {tuple(scales.shape)} != [.., {groups}, {N}]")
+    if tuple(qzeros.shape[lead:]) != (groups, NW):
+        raise ValueError(f"qzeros shape {tuple(qzeros.shape)} != [.., {groups}, {NW}]")
+    if lead and not (qweight.shape[0] == scales.shape[0] == qzeros.shape[0]):
+        raise ValueError("expert dimension differs between qweight / scales / qzeros")
+    return K, N, K // groups
+
+
+def get_workspace(device, nbytes: int) -> torch.Tensor:
+    """Per (device, stream) zero-initialised workspace; the kernels leave the counter
+    prefix zeroed, so it is reused call after call."""
+    dev = torch.device(device)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(dev).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        _workspaces[key] = ws
+    return ws
+
+
+def awq_dequantize(qweight: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor,
+                   split_k_iters: int = 0, thx: int = 0, thy: int = 0) -> torch.Tensor:
+    """fp16 [K, N] = fp16((w - z) * s).  split_k_iters / thx / thy are accepted for
+    signature compatibility and ignored."""
+    _need(qweight, "qweight", torch.int32, 2)
+    _need(scales, "scales", torch.float16, 2)
+    _need(zeros, "zeros", torch.int32, 2)
+    K, N, G = _awq_shapes(qweight, scales, zeros)
+    out = torch.empty((K, N), dtype=torch.float16, device=qweight.device)
+    lib = _lib.load()
+    st = lib.awqmi_dequantize_f16(qweight.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
+                                  out.data_ptr(), K, N, G, _stream_ptr(qweight.device))
+    _lib.check(st, "awq_dequantize")
+    return out
+
+
+def awq_gemm(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
+             qzeros: torch.Tensor, split_k_iters: int = 0, out: torch.Tensor | None = None) -> torch.Tensor:
+    """fp16 [M, N] = input[M, K] @ dequant(qweight, scales, qzeros).  split_k_iters = 0 lets
+    the library choose; values above the library maximum are clamped."""
+    _need(input, "input", torch.float16, 2)
+    _need(qweight, "qweight", torch.int32, 2)
+    _need(scales, "scales", torch.float16, 2)
+    _need(qzeros, "qzeros", torch.int32, 2)
+    K, N, G = _awq_shapes(qweight, scales, qzeros)
+    M = input.shape[0]
+    if input.shape[1] != K:
+        raise ValueError(f"input has K={input.shape[1]}, qweight has K={K}")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=input.device)
+    else:
+        _need(out, "out", torch.float16, 2)
+        if tuple(out.shape) != (M, N):
+            raise ValueError("out has the wrong shape")
+    if M == 0:
+        return out
+    lib = _lib.load()
+    split = max(0, min(int(split_k_iters), 64))
+    nbytes = lib.awqmi_gemm_workspace_bytes(M, K, N, split)
+    ws = get_workspace(input.device, nbytes)
+    st = lib.awqmi_gemm_f16(input.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
+                            out.data_ptr(), ws.data_ptr(), ws.numel(), M, K, N, G, split,
+                            _stream_ptr(input.device))
+    _lib.check(st, "awq_gemm")
+    return out
+
+
+# --------------------------------------------------------------------------- fused MoE
+
+def topk_softmax(gating_output: torch.Tensor, topk: int, renormalize: bool = True):
+    """softmax over experts then top-k.  Returns (topk_weights fp32 [T, k], topk_ids int32)."""
+    _need(gating_output, "gating_output", torch.float32, 2)
+    T, E = gating_output.shape
+    ids = torch.empty((T, topk), dtype=torch.int32, device=gating_output.device)
+    wts = torch.empty((T, topk), dtype=torch.float32, device=gating_output.device)
+    if T == 0:
+        return wts, ids
+    st = _lib.load().awqmi_moe_topk_softmax_f32(gating_output.data_ptr(), T, E, topk, int(renormalize),
+                                                ids.data_ptr(), wts.data_ptr(),
+                                                _stream_ptr(gating_output.device))
+    _lib.check(st, "topk_softmax")
+    return wts, ids
+
+
+def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int):
+    """Returns (sorted_token_ids, expert_ids, num_tokens_post_padded): flat slot indices
+    stably sorted by expert, each expert's run padded to a multiple of block_size with the
+    sentinel topk_ids.numel()."""
+    _need(topk_ids, "topk_ids", torch.int32)
+    n = topk_ids.numel()
+    lib = _lib.load()
+    cap = lib.awqmi_moe_align_capacity(n, num_experts, block_size)
+    dev = topk_ids.device
+    sorted_ids = torch.empty((cap,), dtype=torch.int32, device=dev)
+    expert_ids = torch.empty((cap // block_size,), dtype=torch.int32, device=dev)
+    npp = torch.empty((1,), dtype=torch.int32, device=dev)
+    st = lib.awqmi_moe_align(topk_ids.data_ptr(), n, num_experts, block_size, sorted_ids.data_ptr(),
+                             expert_ids.data_ptr(), npp.data_ptr(), _stream_ptr(dev))
+    _lib.check(st, "moe_align_block_size")
+    return sorted_ids, expert_ids, npp
+
+
+def moe_awq_gemm(a: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, qzeros: torch.Tensor,
+                 sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
+                 num_tokens_post_padded: torch.Tensor, n_slots: int, a_row_div: int,
+                 topk_weights: torch.Tensor | None = None, split_k: int = 0,
+                 out: torch.Tensor | None = None) -> torch.Tensor:
+    """Expert-grouped AWQ GEMM over blocks of 16 sorted slots: out[s] = a[s // a_row_div] @
+    W[expert(s)] (* topk_weights[s])."""
+    _need(a, "a", torch.float16, 2)
+    _need(qweight, "qweight", torch.int32, 3)
+    _need(scales, "scales", torch.float16, 3)
+    _need(qzeros, "qzeros", torch.int32, 3)
+    _need(sorted_token_ids, "sorted_token_ids", torch.int32, 1)
+    _need(expert_ids, "expert_ids", torch.int32, 1)
+    _need(num_tokens_post_padded, "num_tokens_post_padded", torch.int32, 1)
+    K, N, G = _awq_shapes(qweight, scales, qzeros, lead=1)
+    E = qweight.shape[0]
+    if a.shape[1] != K:
+        raise ValueError(f"a has K={a.shape[1]}, qweight has K={K}")
+    if a.shape[0] * a_row_div < n_slots:
+        raise ValueError("a has too few rows for n_slots / a_row_div")
+    lib = _lib.load()
+    cap = lib.awqmi_moe_align_capacity(n_slots, E, MOE_TILE_M)
+    if sorted_token_ids.numel() < cap or expert_ids.numel() < cap // MOE_TILE_M:
+        raise ValueError("sorted_token_ids / expert_ids smaller than the align capacity")
+    tw = 0
+    if topk_weights is not None:
+        _need(topk_weights, "topk_weights", torch.float32)
+        if topk_weights.numel() < n_slots:
+            raise ValueError("topk_weights has fewer entries than n_slots")
+        tw = topk_weights.data_ptr()
+    if out is None:
+        out = torch.empty((n_slots, N), dtype=torch.float16, device=a.device)
+    split = max(0, min(int(split_k), 64))
+    nbytes = lib.awqmi_moe_gemm_workspace_bytes(n_slots, E, K, N, split)
+    ws = get_workspace(a.device, nbytes)
+    st = lib.awqmi_moe_gemm_f16(a.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
+                                out.data_ptr(), sorted_token_ids.data_ptr(), expert_ids.data_ptr(),
+                                num_tokens_post_padded.data_ptr(), tw, n_slots, a_row_div, E, K, N, G,
+                                split, ws.data_ptr(), ws.numel(), _stream_ptr(a.device))
+    _lib.check(st, "moe_awq_gemm")
+    return out
+
+
+def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
+    """[rows, 2I] ([gate | up]) -> silu(gate) * up, fp16 [rows, I]."""
+    _need(x, "x", torch.float16, 2)
+    rows, two_i = x.shape
+    out = torch.empty((rows, two_i // 2), dtype=torch.float16, device=x.device)
+    st = _lib.load().awqmi_silu_and_mul_f16(x.data_ptr(), out.data_ptr(), rows, two_i // 2,
+                                           _stream_ptr(x.device))
+    _lib.check(st, "silu_and_mul")
+    return out
+
+
+def moe_sum(x: torch.Tensor, T: int, topk: int) -> torch.Tensor:
+    """[T * topk, H] -> [T, H], fp32 sum over a token's slots."""
+    _need(x, "x", torch.float16, 2)
+    H = x.shape[1]
+    out = torch.empty((T, H), dtype=torch.float16, device=x.device)
+    st = _lib.load().awqmi_moe_sum_f16(x.data_ptr(), out.data_ptr(), T, topk, H, _stream_ptr(x.device))
+    _lib.check(st, "moe_sum")
+    return out
+
+
+def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Tensor, topk: int,
+                  renormalize: bool = True) -> torch.Tensor:
+    """One AWQ MoE block: route -> align -> grouped GEMM (w13) -> SiLU*up -> grouped GEMM (w2,
+    scaled by the routing weight) -> sum over slots.  w13 / w2 are (qweight, scales, qzeros)
+    with a leading expert dimension; w13 columns are [gate | up]."""
+    T = hidden_states.shape[0]
+    E = w13[0].shape[0]
+    topk_w, topk_ids = topk_softmax(gating_output.float().contiguous(), topk, renormalize)
+    sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, MOE_TILE_M, E)
+    n = T * topk
+    h13 = moe_awq_gemm(hidden_states, *w13, sorted_ids, expert_ids, npp, n, topk)
+    act = silu_and_mul(h13)
+    o = moe_awq_gemm(act, *w2, sorted_ids, expert_ids, npp, n, 1, topk_weights=topk_w)
+    return moe_sum(o, T, topk)

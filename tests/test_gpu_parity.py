@@ -1,0 +1,195 @@
+"""GPU parity: the HIP kernels, called through the C ABI (ctypes), against the CPU oracle on
+the same seeded inputs.  Integer / dequant results must be bit-exact; GEMM outputs must be
+within a relative Frobenius error of 2e-3 of the float64 product of the fp16 inputs and the
+pinned fp16 weights (TOL below), max-abs error printed."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import awq_ref
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _np_case(M, K, N, G, seed):
+    rng = np.random.default_rng(seed)
+    g = K if G <= 0 else G
+    w = rng.integers(0, 16, (K, N))
+    z = rng.integers(0, 16, (K // g, N))
+    s = (rng.random((K // g, N)) * 0.019 + 0.001).astype(np.float16)
+    x = rng.normal(0, 1, (M, K)).astype(np.float16)
+    return x, awq_ref.pack_awq(w), s, awq_ref.pack_awq(z)
+
+
+def _dev(dev, *arrs):
+    return [torch.from_numpy(np.ascontiguousarray(a)).to(dev) for a in arrs]
+
+
+def _check_gemm(sba, dev, x, qw, s, qz, G, split_k=0, tag=""):
+    ref = awq_ref.gemm_wide(x, qw, s, qz, G)
+    xd, qwd, sd, qzd = _dev(dev, x, qw, s, qz)
+    y = sba.awq_gemm(xd, qwd, sd, qzd, split_k)
+    torch.cuda.synchronize()
+    yh = y.cpu().numpy()
+    err = awq_ref.rel_frobenius(yh, ref)
+    maxabs = float(np.max(np.abs(yh.astype(np.float64) - ref)))
+    print(f"[gemm {tag} M={x.shape[0]} K={x.shape[1]} N={qw.shape[1] * 8} G={G} split={split_k}] "
+          f"rel_fro={err:.2e} max_abs={maxabs:.3e}", flush=True)
+    assert np.isfinite(yh).all()
+    assert err <= TOL
+    return yh
+
+
+# ------------------------------------------------------------------ dequantize (bit-exact)
+
+@pytest.mark.parametrize("K,N,G", [(256, 64, 128), (4096, 4096, 128), (128, 8, 32), (96, 40, 24),
+                                   (64, 2056, 64), (384, 128, -1), (30, 16, 3), (512, 264, 256)])
+def test_dequantize_bit_exact(sba, gpu, K, N, G):
+    _, qw, s, qz = _np_case(1, K, N, G, seed=K + N)
+    want = awq_ref.dequantize(qw, s, qz, G)
+    qwd, sd, qzd = _dev(gpu, qw, s, qz)
+    got = sba.awq_dequantize(qwd, sd, qzd, 0, 0, 0).cpu().numpy()
+    assert got.shape == want.shape
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+def test_dequantize_exhaustive_and_fixture(sba, gpu):
+    h = np.arange(65536, dtype=np.uint16).view(np.float16)
+    with np.errstate(invalid="ignore"):
+        finite = h[np.isfinite(h)]
+    # every finite fp16 scale (subnormal results included) x every (w, z) pair
+    S = finite.size
+    N = 16 * S
+    N8 = (N + 7) // 8 * 8
+    w = np.repeat(np.arange(16)[:, None], N8, axis=1)
+    z = np.zeros((1, N8), np.int64)
+    s = np.ones((1, N8), np.float16)
+    for zz in range(16):
+        z[0, zz * S:(zz + 1) * S] = zz
+        s[0, zz * S:(zz + 1) * S] = finite
+    qw, qz = awq_ref.pack_awq(w), awq_ref.pack_awq(z)
+    with np.errstate(over="ignore"):
+        want = ((w - z).astype(np.float64) * s.astype(np.float64)).astype(np.float16)
+    got = sba.awq_dequantize(*_dev(gpu, qw, s, qz), 0, 0, 0).cpu().numpy()
+    gb, wb = got.view(np.uint16), want.view(np.uint16)
+    same = (gb == wb) | (((gb | wb) & 0x7FFF) == 0)     # +0 / -0 both fine
+    assert same.all(), np.argwhere(~same)[:5]
+
+    fx = np.load(os.path.join(GOLDEN, "awq_small.npz"))
+    got = sba.awq_dequantize(*_dev(gpu, fx["qweight"], fx["scales"], fx["qzeros"]), 0, 0, 0).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), fx["w_dequant_bits"])
+
+
+# ------------------------------------------------------------------ decode GEMM (M <= 16)
+
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("M", [1, 4, 8, 16])
+def test_gemm_decode_small(sba, gpu, M, variant):
+    from server_benchmark_amd import _lib
+    lib = _lib.load()
+    prev = lib.awqmi_set_gemv_variant(variant)
+    try:
+        x, qw, s, qz = _np_case(M, 1024, 512, 128, seed=10 + M)
+        for split in (0, 1, 2, 3, 8):
+            _check_gemm(sba, gpu, x, qw, s, qz, 128, split, tag=f"v{variant}")
+    finally:
+        lib.awqmi_set_gemv_variant(prev)
+
+
+@pytest.mark.parametrize("K,N,G", [(256, 128, 32), (256, 264, 64), (512, 136, 256), (384, 8, -1),
+                                   (128, 2048, 128), (640, 1000, 128)])
+def test_gemm_decode_groups_and_ragged_n(sba, gpu, K, N, G):
+    x, qw, s, qz = _np_case(5, K, N, G, seed=K * 3 + N)
+    g = K if G <= 0 else G
+    for split in (0, 1, 2):
+        _check_gemm(sba, gpu, x, qw, s, qz, g, split)
+
+
+def test_gemm_one_hot_is_exact_and_zero_weights(sba, gpu):
+    K, N, G = 512, 256, 128
+    _, qw, s, qz = _np_case(1, K, N, G, seed=77)
+    W = awq_ref.dequantize(qw, s, qz, G)
+    rows = [0, 1, 127, 128, 300, 511, 37, 64, 200, 255, 256, 383, 384, 385, 450, 9]
+    x = np.zeros((16, K), np.float16)
+    for m, k in enumerate(rows):
+        x[m, k] = 1
+    for split in (1, 4):
+        y = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), split).cpu().numpy()
+        for m, k in enumerate(rows):
+            assert np.array_equal(y[m].view(np.uint16), W[k].view(np.uint16)), (split, m, k)
+    # w == z everywhere -> exact zeros
+    zfull = np.repeat(awq_ref.unpack_awq(qz), G, axis=0)
+    xr = np.random.default_rng(0).normal(0, 1, (16, K)).astype(np.float16)
+    y = sba.awq_gemm(*_dev(gpu, xr, awq_ref.pack_awq(zfull), s, qz), 0).cpu().numpy()
+    assert not y.any()
+
+
+def test_gemm_config0(sba, gpu):
+    c = sba.workloads.config0()
+    x, qw, s, qz = (t.numpy() for t in (c.x, c.qweight, c.scales, c.qzeros))
+    y16 = _check_gemm(sba, gpu, x, qw, s, qz, 128, 0, tag="config0")
+    # row 0 alone (M = 1) equals row 0 of the M = 16 run: the kernel does not depend on M
+    y1 = sba.awq_gemm(*_dev(gpu, x[:1], qw, s, qz), 0).cpu().numpy()
+    assert awq_ref.rel_frobenius(y1[0], y16[0]) < 1e-3
+    W = sba.awq_dequantize(*_dev(gpu, qw, s, qz)).cpu().numpy()
+    assert np.array_equal(W.view(np.uint16), awq_ref.dequantize(qw, s, qz, 128).view(np.uint16))
+
+
+def test_gemm_workspace_counters_stay_zero(sba, gpu):
+    from server_benchmark_amd import ops
+    x, qw, s, qz = _np_case(16, 1024, 512, 128, seed=3)
+    d = _dev(gpu, x, qw, s, qz)
+    for _ in range(3):
+        sba.awq_gemm(*d, 4)
+    torch.cuda.synchronize()
+    ws = ops.get_workspace(gpu, 1)
+    assert int(ws[:65536].view(torch.int32).abs().sum().item()) == 0
+
+
+# ------------------------------------------------------------------ prefill GEMM (M > 16) and fallback
+
+@pytest.mark.parametrize("M,K,N,G", [(17, 256, 256, 128), (64, 512, 512, 128), (300, 1024, 520, 128),
+                                     (512, 2048, 1024, 128), (257, 192, 264, 32), (40, 256, 128, 64),
+                                     (33, 384, 256, -1)])
+def test_gemm_prefill(sba, gpu, M, K, N, G):
+    x, qw, s, qz = _np_case(M, K, N, G, seed=M + K)
+    _check_gemm(sba, gpu, x, qw, s, qz, K if G <= 0 else G, 0, tag="prefill")
+
+
+@pytest.mark.parametrize("M,K,N,G", [(3, 96, 40, 32), (20, 100, 16, 50), (2, 24, 8, 8)])
+def test_gemm_generic_fallback(sba, gpu, M, K, N, G):
+    x, qw, s, qz = _np_case(M, K, N, G, seed=5)
+    _check_gemm(sba, gpu, x, qw, s, qz, G, 0, tag="generic")
+
+
+def test_bad_arguments_raise_without_launch(sba, gpu):
+    x, qw, s, qz = _dev(gpu, *_np_case(2, 256, 64, 128, seed=1))
+    with pytest.raises(ValueError):
+        sba.awq_gemm(x[:, :128].contiguous(), qw, s, qz, 0)
+    with pytest.raises(ValueError):
+        sba.awq_gemm(x.float(), qw, s, qz, 0)
+    with pytest.raises(ValueError):
+        sba.awq_gemm(x.cpu(), qw, s, qz, 0)
+    with pytest.raises(ValueError):
+        sba.awq_dequantize(qw, s[:, :32].contiguous(), qz)
+
+
+def test_linear_method_apply(sba, gpu):
+    cfg = sba.AWQConfig.from_config({"w_bit": 4, "q_group_size": 128, "zero_point": True})
+    layer = torch.nn.Module()
+    m = cfg.get_quant_method(layer, "model.layers.0.mlp.down_proj")
+    m.create_weights(layer, 512, [128, 128], 512, 256, torch.float16, device=gpu)
+    x, qw, s, qz = _np_case(6, 512, 256, 128, seed=9)
+    sd = {"qweight": torch.from_numpy(qw), "qzeros": torch.from_numpy(qz), "scales": torch.from_numpy(s)}
+    layer.load_state_dict(sd)
+    m.process_weights_after_loading(layer)
+    xin = torch.from_numpy(x).to(gpu).reshape(2, 3, 512)
+    bias = torch.linspace(-1, 1, 256, dtype=torch.float16, device=gpu)
+    y = m.apply(layer, xin, bias)
+    assert y.shape == (2, 3, 256)
+    ref = awq_ref.gemm_wide(x, qw, s, qz, 128) + bias.cpu().numpy().astype(np.float64)
+    assert awq_ref.rel_frobenius(y.reshape(6, 256).cpu().numpy(), ref) <= TOL
