@@ -1,0 +1,292 @@
+#!/usr/bin/env python3
+"""Benchmark of the AWQ W4A16 linear path on one MI355X.
+
+A "step" is one pass of the decode sweep the metric is quoted on: the four Qwen2.5-72B AWQ
+linears (qkv_proj, o_proj, gate_up_proj, down_proj; group 128) at M in {1, 4, 8, 16} fp16
+tokens, 16 launches of awq_gemm through the C ABI.  Inputs are resident in HBM before the
+timed region.  Every layer keeps four distinct weight copies and the M-th launch of a layer
+uses copy M, so between two uses of the same buffer ~1.8 GB of other weights stream through
+and the 256 MB Infinity Cache cannot serve them: the reported figure is HBM bandwidth.
+
+`value` = algorithmic bytes of a step (packed weights + scales + packed zeros + activations
+in + out) / time per step.  The prefill sweep (M in {512, 2048, 8192}, fp16 MFMA TFLOP/s) is
+measured after the timed region and reported under "prefill".  The CPU baseline leg times
+the PyTorch dequantize-then-matmul oracle on the host cores over a bounded sample.
+
+Prints ONE JSON line on stdout; progress goes to stderr.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_weights(K, N, G, device, gen):
+    import torch
+    lo, hi = -(2 ** 31), 2 ** 31
+    qw = torch.randint(lo, hi, (K, N // 8), dtype=torch.int32, device=device, generator=gen)
+    qz = torch.randint(lo, hi, (K // G, N // 8), dtype=torch.int32, device=device, generator=gen)
+    sc = (torch.rand((K // G, N), device=device, generator=gen) * 0.019 + 0.001).to(torch.float16)
+    return qw, sc, qz
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--launch", choices=("graph", "direct"), default="graph",
+                    help="replay the step as a HIP graph (how a serving engine decodes) or launch directly")
+    ap.add_argument("--split-k", type=int, default=0, help="0 = library heuristic")
+    ap.add_argument("--variant", type=int, default=-1, help="development: skinny-kernel variant")
+    ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--detail", action="store_true", help="per-point timings on stderr")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        log("bench.py: this build measures one GPU only (the path shards without changing the "
+            "kernel; see DESIGN.md).  Run with --gpus 1.")
+        sys.exit(2)
+
+    import torch
+    sba = __import__("server_benchmark_amd")
+    from server_benchmark_amd import _lib, workloads
+
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible; the HIP path has no CPU fallback")
+        sys.exit(1)
+    lib = _lib.load()
+    if args.variant >= 0:
+        lib.awqmi_set_gemv_variant(args.variant)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    G = 128
+    layers = workloads.QWEN25_72B_LAYERS
+    Ms = workloads.DECODE_M
+    NCOPY = len(Ms)
+
+    t0 = time.time()
+    W = {}
+    X = {}
+    Y = {}
+    for name, K, N in layers:
+        W[name] = [make_weights(K, N, G, dev, gen) for _ in range(NCOPY)]
+        X[name] = {M: torch.randn((M, K), device=dev, generator=gen).to(torch.float16) for M in Ms}
+        Y[name] = {M: torch.empty((M, N), dtype=torch.float16, device=dev) for M in Ms}
+    ws_bytes = max(lib.awqmi_gemm_workspace_bytes(M, K, N, args.split_k) for _, K, N in layers for M in Ms)
+    ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
+    torch.cuda.synchronize()
+    log(f"[bench] inputs resident after {time.time() - t0:.1f}s, "
+        f"{torch.cuda.memory_allocated() / 2**30:.2f} GiB allocated")
+
+    def launch(name, K, N, M, copy, stream_ptr):
+        qw, sc, qz = W[name][copy]
+        st = lib.awqmi_gemm_f16(X[name][M].data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(),
+                                Y[name][M].data_ptr(), ws.data_ptr(), ws.numel(), M, K, N, G,
+                                args.split_k, stream_ptr)
+        if st != 0:
+            raise RuntimeError(f"awqmi_gemm_f16 failed: {lib.awqmi_status_string(st).decode()}")
+
+    def step(stream_ptr):
+        for ci, M in enumerate(Ms):
+            for name, K, N in layers:
+                launch(name, K, N, M, ci, stream_ptr)
+
+    step_bytes = sum(workloads.linear_bytes(M, K, N, G) for _, K, N in layers for M in Ms)
+    n_launch = len(layers) * len(Ms)
+
+    graph = None
+    if args.launch == "graph":
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step(side.cuda_stream)          # warm the code objects outside capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step(torch.cuda.current_stream().cuda_stream)
+
+    def run_step():
+        if graph is not None:
+            graph.replay()
+        else:
+            step(torch.cuda.current_stream().cuda_stream)
+
+    for _ in range(args.warmup):
+        run_step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t_start = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        run_step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t_start
+    ev_ms = e0.elapsed_time(e1)
+    ms_per_step = wall * 1e3 / args.steps
+    value = step_bytes / (wall / args.steps) / 1e9
+    kern_avg_us = ev_ms * 1e3 / (args.steps * n_launch)
+    achieved = step_bytes / n_launch / (kern_avg_us * 1e-6) / 1e9
+    log(f"[bench] decode sweep: {ms_per_step:.3f} ms/step wall, {ev_ms / args.steps:.3f} ms/step events, "
+        f"{value:.0f} GB/s ({value / HBM_PEAK_GBS:.1%} of {HBM_PEAK_GBS:.0f})")
+
+    # per-point detail (direct launches, event pair per point, same rotation)
+    points = []
+    stream_ptr = torch.cuda.current_stream().cuda_stream
+    reps = 10
+    for name, K, N in layers:
+        for ci, M in enumerate(Ms):
+            # flush the last-level cache with the other layers' copies between points
+            evs = []
+            for r in range(reps):
+                for oname, oK, oN in layers:
+                    if oname != name:
+                        launch(oname, oK, oN, 16, (ci + r) % NCOPY, stream_ptr)
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                launch(name, K, N, M, (ci + r) % NCOPY, stream_ptr)
+                b.record()
+                evs.append((a, b))
+            torch.cuda.synchronize()
+            ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)
+            med = ts[len(ts) // 2]
+            nbytes = workloads.linear_bytes(M, K, N, G)
+            points.append({"layer": name, "M": M, "K": K, "N": N, "us": round(med, 2),
+                           "GBps": round(nbytes / med / 1e3, 1),
+                           "frac_hbm": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4),
+                           "split_k": lib.awqmi_gemm_auto_split_k(M, K, N, G) if args.split_k == 0 else args.split_k})
+            if args.detail:
+                log(f"   {name:13s} M={M:2d}  {med:8.2f} us  {nbytes / med / 1e3:8.1f} GB/s")
+
+    out = {
+        "metric": "AWQ W4A16 GEMM HBM GB/s (decode) & TFLOP/s (prefill), 72B shapes, 1 GPU",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int4 weights x fp16 activations, fp32 accumulate",
+        "data": "synthetic: on-device seeded uniform int4 weights/zeros in AWQ packing, "
+                "U[0.001,0.02] fp16 scales, N(0,1) fp16 activations",
+        "config": {"workload": "decode GEMV sweep, Qwen2.5-72B AWQ layer shapes (qkv 8192x10240, o 8192x8192, "
+                               "gate_up 8192x59136, down 29568x8192), group 128, M in {1,4,8,16}; "
+                               "16 awq_gemm launches per step, 4 rotating weight copies per layer",
+                   "launch": args.launch, "split_k": args.split_k, "bytes_per_step": step_bytes},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "awq_gemv_kernel", "avg_launch_us": round(kern_avg_us, 2),
+                     "bytes_per_launch": step_bytes // n_launch},
+        "decode_points": points,
+    }
+
+    # ------------------------------------------------------------------ prefill sweep
+    if not args.no_prefill:
+        pts = []
+        tot_f, tot_t = 0.0, 0.0
+        for name, K, N in layers:
+            qw, sc, qz = W[name][0]
+            for M in workloads.PREFILL_M:
+                x = torch.randn((M, K), device=dev, generator=gen).to(torch.float16)
+                y = torch.empty((M, N), dtype=torch.float16, device=dev)
+
+                def call():
+                    st = lib.awqmi_gemm_f16(x.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(),
+                                            y.data_ptr(), ws.data_ptr(), ws.numel(), M, K, N, G, 0, stream_ptr)
+                    if st != 0:
+                        raise RuntimeError(lib.awqmi_status_string(st).decode())
+
+                call()
+                call()
+                torch.cuda.synchronize()
+                n_it = 3 if M >= 8192 else 6
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                for _ in range(n_it):
+                    call()
+                b.record()
+                torch.cuda.synchronize()
+                ms = a.elapsed_time(b) / n_it
+                fl = workloads.linear_flops(M, K, N)
+                tf = fl / ms / 1e9
+                tot_f += fl
+                tot_t += ms
+                pts.append({"layer": name, "M": M, "ms": round(ms, 4), "TFLOPs": round(tf, 1),
+                            "frac_mfma": round(tf / MFMA_FP16_PEAK_TFLOPS, 4)})
+                if args.detail:
+                    log(f"   prefill {name:13s} M={M:5d} {ms:9.3f} ms {tf:8.1f} TFLOP/s")
+                del x, y
+        agg = tot_f / tot_t / 1e9
+        out["prefill"] = {"unit": "TFLOP/s", "aggregate": round(agg, 1), "peak": MFMA_FP16_PEAK_TFLOPS,
+                          "frac": round(agg / MFMA_FP16_PEAK_TFLOPS, 4), "kernel": "awq_gemm_mfma_kernel",
+                          "points": pts}
+        log(f"[bench] prefill sweep aggregate {agg:.1f} TFLOP/s ({agg / MFMA_FP16_PEAK_TFLOPS:.1%} of fp16 MFMA peak)")
+
+    # ------------------------------------------------------------------ CPU baseline leg
+    if not args.no_cpu:
+        from oracle import awq_ref   # the checker: timed here as the reference CPU path
+        ncores = os.cpu_count() or 1
+        nthreads = min(ncores, int(os.environ.get("OMP_NUM_THREADS", ncores)))
+        torch.set_num_threads(nthreads)
+        name, K, N = layers[0]
+        qw, sc, qz = (t.cpu() for t in W[name][0])
+        sample_bytes, sample_t = 0, 0.0
+        worst = 0.0
+        awq_ref.cpu_linear_torch(X[name][1].cpu(), qw, sc, qz, G)      # warm-up
+        for M in Ms:
+            xc = X[name][M].cpu()
+            t1 = time.perf_counter()
+            yc = awq_ref.cpu_linear_torch(xc, qw, sc, qz, G)
+            sample_t += time.perf_counter() - t1
+            sample_bytes += workloads.linear_bytes(M, K, N, G)
+            # the same call on the GPU must agree with the CPU path (checker)
+            yg = sba.awq_gemm(X[name][M], *W[name][0], 0).float().cpu()
+            err = float((yg - yc.float()).norm() / yc.float().norm())
+            worst = max(worst, err)
+        cpu_model = ""
+        try:
+            with open("/proc/cpuinfo") as f:
+                for line in f:
+                    if line.startswith("model name"):
+                        cpu_model = line.split(":", 1)[1].strip()
+                        break
+        except OSError:
+            pass
+        out["cpu_baseline"] = {"value": round(sample_bytes / sample_t / 1e9, 3), "unit": "GB/s",
+                               "cores": nthreads, "kind": "port",
+                               "sample": f"{name} K={K} N={N} at M in {list(Ms)}, one PyTorch "
+                                         f"dequantize+matmul call each ({sample_t:.1f} s total)",
+                               "cpu": cpu_model, "gpu_vs_cpu_rel_frobenius_max": round(worst, 6)}
+        log(f"[bench] cpu baseline {out['cpu_baseline']['value']} GB/s on {nthreads} threads; "
+            f"GPU vs CPU rel. Frobenius max {worst:.2e}")
+        if worst > 2e-3:
+            log("[bench] ERROR: GPU result differs from the CPU path beyond 2e-3")
+            print(json.dumps(out))
+            sys.exit(1)
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,189 @@
+"""CPU-only checks of the host side: the C-ABI library loads and exports every symbol the
+header declares, host-side validation rejects bad calls before any launch, the layer
+methods register the right parameters, and the workload generators produce the stated
+shapes and byte counts.  No compute call is made (no GPU here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from server_benchmark_amd import _lib
+    return _lib.load()
+
+
+def test_library_exports_every_declared_symbol(lib):
+    from server_benchmark_amd import _lib
+    hdr = open(os.path.join(ROOT, "include", "awq_mi355x.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    declared = set(re.findall(r"\b(awqmi_[a-z0-9_]+)\s*\(", hdr))
+    assert len(declared) >= 14
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    assert lib.awqmi_version() == 100
+
+
+def test_status_strings(lib):
+    seen = {lib.awqmi_status_string(i).decode() for i in range(8)}
+    assert len(seen) == 8 and "ok" in seen
+    assert lib.awqmi_status_string(99).decode() == "unknown status"
+
+
+def test_validation_happens_before_any_launch(lib):
+    fake = 0x1000   # non-null, 16-byte aligned, never dereferenced on these paths
+    odd = 0x1008
+    # null pointers
+    assert lib.awqmi_dequantize_f16(0, fake, fake, fake, 128, 64, 128, 0) == 6
+    assert lib.awqmi_gemm_f16(fake, fake, fake, fake, 0, 0, 0, 1, 128, 64, 128, 0, 0) == 6
+    # shape relations: N % 8, K % group, positive sizes
+    assert lib.awqmi_dequantize_f16(fake, fake, fake, fake, 128, 60, 128, 0) == 1
+    assert lib.awqmi_dequantize_f16(fake, fake, fake, fake, 100, 64, 48, 0) == 1
+    assert lib.awqmi_gemm_f16(fake, fake, fake, fake, fake, 0, 0, 0, 128, 64, 128, 0, 0) == 1
+    assert lib.awqmi_gemm_f16(fake, fake, fake, fake, fake, 0, 0, 4, 128, 64, 96, 0, 0) == 1
+    # alignment
+    assert lib.awqmi_dequantize_f16(fake, odd, fake, fake, 128, 64, 128, 0) == 2
+    assert lib.awqmi_gemm_f16(odd, fake, fake, fake, fake, 0, 0, 4, 128, 64, 128, 0, 0) == 2
+    # split_k range, missing / short workspace
+    assert lib.awqmi_gemm_f16(fake, fake, fake, fake, fake, 0, 0, 4, 1024, 64, 128, 65, 0) == 7
+    assert lib.awqmi_gemm_f16(fake, fake, fake, fake, fake, 0, 0, 4, 1024, 64, 128, 2, 0) == 6
+    assert lib.awqmi_gemm_f16(fake, fake, fake, fake, fake, fake, 1000, 4, 1024, 64, 128, 2, 0) == 3
+    # MoE entry points
+    assert lib.awqmi_moe_align(0, 8, 4, 16, fake, fake, fake, 0) == 6
+    assert lib.awqmi_moe_align(fake, 8, 2000, 16, fake, fake, fake, 0) == 7
+    assert lib.awqmi_moe_topk_softmax_f32(fake, 4, 8, 9, 1, fake, fake, 0) == 7
+    assert lib.awqmi_moe_gemm_f16(fake, fake, fake, fake, fake, fake, fake, fake, 0, 8, 2, 4, 100, 64, 50,
+                                  0, 0, 0, 0) == 4
+    assert lib.awqmi_silu_and_mul_f16(fake, fake, 4, 12, 0) == 1
+    assert lib.awqmi_moe_sum_f16(fake, fake, 4, 2, 12, 0) == 1
+
+
+def test_workspace_and_split_k_queries(lib):
+    for M, K, N in [(1, 8192, 10240), (16, 8192, 8192), (16, 8192, 59136), (4, 29568, 8192), (8, 4096, 4096)]:
+        s = lib.awqmi_gemm_auto_split_k(M, K, N, 128)
+        assert 1 <= s <= 64 and s <= K // 128
+        need = lib.awqmi_gemm_workspace_bytes(M, K, N, 0)
+        assert need == lib.awqmi_gemm_workspace_bytes(M, K, N, s)
+        assert need >= 65536
+        if s > 1:
+            assert need >= 65536 + s * 16 * N * 4
+    assert lib.awqmi_gemm_workspace_bytes(512, 8192, 8192, 0) == 65536      # MFMA kernel: no partials
+    assert lib.awqmi_gemm_auto_split_k(512, 8192, 8192, 128) == 1
+    assert lib.awqmi_moe_align_capacity(8, 128, 16) == (8 + 128 * 15 + 15) // 16 * 16
+    assert lib.awqmi_moe_align_capacity(4096, 128, 16) % 16 == 0
+
+
+def test_ops_reject_cpu_tensors_and_bad_dtypes(sba):
+    c = sba.workloads.make_linear_case(2, 256, 64, 128, seed=0)
+    with pytest.raises(ValueError, match="GPU"):
+        sba.awq_gemm(c.x, c.qweight, c.scales, c.qzeros, 0)
+    with pytest.raises(ValueError, match="GPU"):
+        sba.awq_dequantize(c.qweight, c.scales, c.qzeros, 0, 0, 0)
+    with pytest.raises(ValueError):
+        sba.awq_gemm(c.x.float(), c.qweight, c.scales, c.qzeros, 0)
+    with pytest.raises(TypeError):
+        sba.awq_gemm(c.x.numpy(), c.qweight, c.scales, c.qzeros, 0)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from server_benchmark_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no CPU or eager fallback"):
+        _lib.load()
+
+
+# ------------------------------------------------------------------ AWQConfig / layer methods
+
+@pytest.mark.parametrize("cfg,want", [
+    ({"w_bit": 4, "q_group_size": 128, "zero_point": True}, (4, 128, True)),
+    ({"bits": 4, "group_size": 64, "zero_point": False}, (4, 64, False)),
+    ({"bits": 4, "group_size": -1, "zero_point": True, "modules_to_not_convert": ["lm_head"]}, (4, -1, True)),
+])
+def test_awq_config_aliases(sba, cfg, want):
+    c = sba.AWQConfig.from_config(cfg)
+    assert (c.weight_bits, c.group_size, c.zero_point) == want
+    assert c.pack_factor == 8 and c.get_name() == "awq"
+    assert torch.float16 in c.get_supported_act_dtypes()
+
+
+def test_awq_config_rejects(sba):
+    with pytest.raises(ValueError):
+        sba.AWQConfig.from_config({"bits": 8, "group_size": 128, "zero_point": True})
+    with pytest.raises(ValueError):
+        sba.AWQConfig.from_config({"group_size": 128, "zero_point": True})
+    c = sba.AWQConfig(4, 128, True, ["lm_head", "gate"])
+    assert c.get_quant_method(torch.nn.Module(), "model.lm_head") is None
+    assert isinstance(c.get_quant_method(torch.nn.Module(), "model.layers.0.self_attn.qkv_proj"),
+                      sba.AWQLinearMethod)
+    moe = torch.nn.Module()
+    moe.is_fused_moe = True
+    assert isinstance(c.get_quant_method(moe, "model.layers.0.mlp.experts"), sba.AWQMoEMethod)
+
+
+def test_linear_method_create_weights(sba):
+    cfg = sba.AWQConfig(4, 128, True)
+    m = sba.AWQLinearMethod(cfg)
+    layer = torch.nn.Module()
+    m.create_weights(layer, 8192, [8192, 1024, 1024], 8192, 10240, torch.float16, weight_loader="wl")
+    assert tuple(layer.qweight.shape) == (8192, 1280) and layer.qweight.dtype == torch.int32
+    assert tuple(layer.qzeros.shape) == (64, 1280) and layer.qzeros.dtype == torch.int32
+    assert tuple(layer.scales.shape) == (64, 10240) and layer.scales.dtype == torch.float16
+    assert layer.qweight.packed_dim == 1 and layer.qweight.pack_factor == 8
+    assert layer.qweight.weight_loader == "wl"
+    assert sorted(n for n, _ in layer.named_parameters()) == ["qweight", "qzeros", "scales"]
+    with pytest.raises(ValueError, match="input size"):
+        m.create_weights(torch.nn.Module(), 8192 + 64, [1024], 8256, 1024, torch.float16)
+    with pytest.raises(ValueError, match="output size"):
+        m.create_weights(torch.nn.Module(), 8192, [1020], 8192, 1020, torch.float16)
+    m1 = sba.AWQLinearMethod(sba.AWQConfig(4, -1, True))
+    l1 = torch.nn.Module()
+    m1.create_weights(l1, 512, [256], 512, 256, torch.float16)
+    assert tuple(l1.scales.shape) == (1, 256)
+
+
+def test_moe_method_create_weights(sba):
+    m = sba.AWQMoEMethod(sba.AWQConfig(4, 128, True))
+    layer = torch.nn.Module()
+    m.create_weights(layer, 128, 2048, 768, torch.float16)
+    assert tuple(layer.w13_qweight.shape) == (128, 2048, 192)
+    assert tuple(layer.w13_scales.shape) == (128, 16, 1536)
+    assert tuple(layer.w13_qzeros.shape) == (128, 16, 192)
+    assert tuple(layer.w2_qweight.shape) == (128, 768, 256)
+    assert tuple(layer.w2_scales.shape) == (128, 6, 2048)
+    assert tuple(layer.w2_qzeros.shape) == (128, 6, 256)
+
+
+# ------------------------------------------------------------------ workloads
+
+def test_workload_shapes_and_bytes(sba):
+    w = sba.workloads
+    c = w.config0()
+    assert tuple(c.x.shape) == (16, 4096) and c.x.dtype == torch.float16
+    assert tuple(c.qweight.shape) == (4096, 512) and tuple(c.qzeros.shape) == (32, 512)
+    assert tuple(c.scales.shape) == (32, 4096)
+    assert float(c.scales.min()) >= 0.001 - 1e-6 and float(c.scales.max()) <= 0.02 + 1e-5
+    c2 = w.config0()
+    assert torch.equal(c.qweight, c2.qweight) and torch.equal(c.x, c2.x)      # seeded
+    # algorithmic byte counts of the benchmark definition
+    assert w.linear_bytes(1, 8192, 10240) == 43_618_304
+    assert w.linear_bytes(16, 8192, 10240) == 44_171_264
+    assert w.linear_bytes(1, 8192, 8192) == 34_897_920
+    assert w.linear_bytes(16, 8192, 59136) == 253_837_312
+    assert w.linear_bytes(4, 29568, 8192) == 126_143_488
+    assert w.linear_bytes(16, 4096, 4096) == 8_978_432
+    assert w.moe_bytes(1, 0, 2048, 768) == 2_451_456
+    assert w.linear_flops(512, 8192, 10240) == 2 * 512 * 8192 * 10240
+
+
+def test_workload_pack_matches_oracle(sba):
+    from oracle import awq_ref
+    v = torch.randint(0, 16, (5, 64), generator=torch.Generator().manual_seed(1))
+    assert np.array_equal(sba.workloads.pack_int4_awq(v).numpy(), awq_ref.pack_awq(v.numpy()))
