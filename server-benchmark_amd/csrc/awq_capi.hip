@@ -51,26 +51,21 @@ inline int gemv_wpl(int N) {
   return (want1 || (N / 8) % 2 != 0) ? 1 : 2;
 }
 
-// Cost model for split-K: bytes moved (weights + fp32 partials out and back) divided by the
-// fraction of the chip's wave slots the launch fills.
+// Split-K choice.  The skinny kernel runs one workgroup (one wave per SIMD, 16 KiB of loads
+// in flight per wave) per CU, and that already saturates HBM; a second round of workgroups
+// costs a drain and refill of the memory pipeline.  So: split K just far enough that the
+// launch is a single round of about 256 workgroups, never below one 128-row chunk per wave.
 int pick_split_k(int rows, int K, int N, int G, long long blocks_z) {
+  (void)rows; (void)G;
   const int nchunks = K / 128;
-  const int ncb = (N + 255) / 256;
-  const double wbytes = (double)K * N / 2.0 * (double)blocks_z;
-  int best = 1;
-  double best_cost = 1e300;
-  const int max_split = nchunks < AWQMI_MAX_SPLIT_K ? nchunks : AWQMI_MAX_SPLIT_K;
-  for (int s = 1; s <= max_split; ++s) {
-    const double waves = (double)ncb * blocks_z * 4.0 * s;
-    const double fill = waves >= 2048.0 ? 1.0 : waves / 2048.0;
-    const double pbytes = s > 1 ? 2.0 * s * rows * (double)N * 4.0 * blocks_z : 0.0;
-    // a wave with under one chunk of work is pure overhead
-    const double idle = (4.0 * s > nchunks) ? (4.0 * s) / nchunks : 1.0;
-    const double cost = (wbytes + pbytes) / fill * idle;
-    if (cost < best_cost * 0.999) { best_cost = cost; best = s; }
-  }
-  (void)G;
-  return best;
+  const long long ncb = (N + 255) / 256;
+  const long long wg = ncb * blocks_z;            // workgroups at split 1
+  long long s = (256 + wg / 2) / wg;              // nearest to one workgroup per CU
+  const long long max_split = nchunks / 4 > 0 ? nchunks / 4 : 1;
+  if (s > max_split) s = max_split;
+  if (s > AWQMI_MAX_SPLIT_K) s = AWQMI_MAX_SPLIT_K;
+  if (s < 1) s = 1;
+  return (int)s;
 }
 
 inline size_t gemv_partial_bytes(int N, int split, long long blocks_z) {

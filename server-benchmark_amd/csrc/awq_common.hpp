@@ -32,6 +32,21 @@ __device__ __forceinline__ uint32_t as_u32(h2 v) { return __builtin_bit_cast(uin
 __device__ __forceinline__ h8 as_h8(u4v v) { return __builtin_bit_cast(h8, v); }
 __device__ __forceinline__ u4v as_u4(h8 v) { return __builtin_bit_cast(u4v, v); }
 
+// Nibble masks held in VGPRs on purpose: with the mask in a register and the magic constant
+// in an SGPR, (t & mask) | magic is a single v_and_or_b32 (a VOP3 op may read one scalar
+// constant only); as literals the compiler has to emit v_and + v_or.
+struct NibbleMasks {
+  uint32_t lo, hi;
+  __device__ __forceinline__ void init() {
+    asm volatile("v_mov_b32 %0, 0x000f000f" : "=v"(lo));
+    asm volatile("v_mov_b32 %0, 0x00f000f0" : "=v"(hi));
+  }
+};
+
+// packed fp16 subtract / multiply on raw 32-bit lanes (v_pk_add_f16 / v_pk_mul_f16)
+__device__ __forceinline__ uint32_t pk_sub(uint32_t a, uint32_t b) { return as_u32(as_h2(a) - as_h2(b)); }
+__device__ __forceinline__ uint32_t pk_mul(uint32_t a, uint32_t b) { return as_u32(as_h2(a) * as_h2(b)); }
+
 // logical column (0..7) held by nibble `nib` of a packed word
 __host__ __device__ constexpr int awq_col_of_nibble(int nib) {
   return nib < 4 ? 2 * nib : 2 * (nib - 4) + 1;

@@ -65,6 +65,8 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+  NibbleMasks nm;
+  nm.init();
   u4v areg[8];
   uint32_t wreg[8];
   uint32_t zreg;
@@ -89,23 +91,23 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   auto dq_byte = [&](half_t* bs, auto BTAG) {
     constexpr int B = decltype(BTAG)::value;
     const uint32_t tz = byte_pair<B>(zreg, zreg);
-    const uint32_t zl = (tz & MASK_LO) | MAGIC_LO, zh = (tz & MASK_HI) | MAGIC_HI;
+    const uint32_t zl = (tz & nm.lo) | MAGIC_LO, zh = (tz & nm.hi) | MAGIC_HI;
+    constexpr int cl = awq_col_of_nibble(2 * B), ch = awq_col_of_nibble(2 * B + 1);
+    // scale of the column in both half-words
+    const uint32_t sw_l = sreg[cl >> 1], sw_h = sreg[ch >> 1];
+    const uint32_t sl = (cl & 1) ? __builtin_amdgcn_perm(sw_l, sw_l, 0x03020302u)
+                                 : __builtin_amdgcn_perm(sw_l, sw_l, 0x01000100u);
+    const uint32_t sh = (ch & 1) ? __builtin_amdgcn_perm(sw_h, sw_h, 0x03020302u)
+                                 : __builtin_amdgcn_perm(sw_h, sw_h, 0x01000100u);
     u4v lo, hi;
 #pragma unroll
     for (int rp = 0; rp < 4; ++rp) {
       const uint32_t t = byte_pair<B>(wreg[2 * rp + 1], wreg[2 * rp]);
-      lo[rp] = (t & MASK_LO) | MAGIC_LO;
-      hi[rp] = (t & MASK_HI) | MAGIC_HI;
+      lo[rp] = pk_mul(pk_sub((t & nm.lo) | MAGIC_LO, zl), sl);
+      hi[rp] = pk_mul(pk_sub((t & nm.hi) | MAGIC_HI, zh), sh);
     }
-    constexpr int cl = awq_col_of_nibble(2 * B), ch = awq_col_of_nibble(2 * B + 1);
-    const h8 sv = as_h8(sreg);
-    const half_t sl = sv[cl], sh = sv[ch];
-    const h8 sl8 = {sl, sl, sl, sl, sl, sl, sl, sl};
-    const h8 sh8 = {sh, sh, sh, sh, sh, sh, sh, sh};
-    const h8 blo = (as_h8(lo) - as_h8(u4v{zl, zl, zl, zl})) * sl8;
-    const h8 bhi = (as_h8(hi) - as_h8(u4v{zh, zh, zh, zh})) * sh8;
-    *reinterpret_cast<h8*>(bs + (8 * wcl + cl) * PF_LD + 8 * kk) = blo;
-    *reinterpret_cast<h8*>(bs + (8 * wcl + ch) * PF_LD + 8 * kk) = bhi;
+    *reinterpret_cast<u4v*>(bs + (8 * wcl + cl) * PF_LD + 8 * kk) = lo;
+    *reinterpret_cast<u4v*>(bs + (8 * wcl + ch) * PF_LD + 8 * kk) = hi;
   };
 
   auto sstore = [&](int buf) {

@@ -39,6 +39,18 @@ struct GemvParams {
   long long w_stride, s_stride, z_stride;  // elements per expert
 };
 
+typedef float f2 __attribute__((ext_vector_type(2)));
+
+// 8-byte device-coherent store / load (relaxed, agent scope)
+__device__ __forceinline__ void st_coherent(float* p, f2 v) {
+  __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), __builtin_bit_cast(unsigned long long, v),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f2 ld_coherent(const float* p) {
+  return __builtin_bit_cast(f2, __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p),
+                                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+
 template <int WPL>
 struct WordVec;
 template <>
@@ -73,10 +85,14 @@ struct GemvWave {
   qvec zcur, znext;
   u4v scur[WPL], snext[WPL];
   uint32_t zlo[WPL][4], zhi[WPL][4];  // (1024+z, 1024+z) / (64+z, 64+z) per byte of the word
+  NibbleMasks nm;
 
   __device__ __forceinline__ GemvWave(const GemvParams& pp) : p(pp) {}
 
   __device__ __forceinline__ void issue(int s, int c) {
+#ifdef AWQMI_LAB_CHUNK_MASK   // lab only: alias all chunks onto a few, so loads hit in L2
+    c &= AWQMI_LAB_CHUNK_MASK;
+#endif
     const size_t row0 = (size_t)c * 128 + 32 * s + 8 * h;
     const qvec* src = reinterpret_cast<const qvec*>(qw + row0 * p.NW);
     const size_t stride = (size_t)p.NW / WPL;
@@ -96,26 +112,26 @@ struct GemvWave {
     for (int w = 0; w < WPL; ++w) {
       const uint32_t zw = WordVec<WPL>::get(zcur, w);
       uint32_t t;
-      t = byte_pair<0>(zw, zw); zlo[w][0] = (t & MASK_LO) | MAGIC_LO; zhi[w][0] = (t & MASK_HI) | MAGIC_HI;
-      t = byte_pair<1>(zw, zw); zlo[w][1] = (t & MASK_LO) | MAGIC_LO; zhi[w][1] = (t & MASK_HI) | MAGIC_HI;
-      t = byte_pair<2>(zw, zw); zlo[w][2] = (t & MASK_LO) | MAGIC_LO; zhi[w][2] = (t & MASK_HI) | MAGIC_HI;
-      t = byte_pair<3>(zw, zw); zlo[w][3] = (t & MASK_LO) | MAGIC_LO; zhi[w][3] = (t & MASK_HI) | MAGIC_HI;
+      t = byte_pair<0>(zw, zw); zlo[w][0] = (t & nm.lo) | MAGIC_LO; zhi[w][0] = (t & nm.hi) | MAGIC_HI;
+      t = byte_pair<1>(zw, zw); zlo[w][1] = (t & nm.lo) | MAGIC_LO; zhi[w][1] = (t & nm.hi) | MAGIC_HI;
+      t = byte_pair<2>(zw, zw); zlo[w][2] = (t & nm.lo) | MAGIC_LO; zhi[w][2] = (t & nm.hi) | MAGIC_HI;
+      t = byte_pair<3>(zw, zw); zlo[w][3] = (t & nm.lo) | MAGIC_LO; zhi[w][3] = (t & nm.hi) | MAGIC_HI;
     }
   }
 
   template <int B>
   __device__ __forceinline__ void tile_pair(int s, int w, bool first) {
     u4v lo, hi;
+    const uint32_t zl = zlo[w][B], zh = zhi[w][B];
 #pragma unroll
     for (int rp = 0; rp < 4; ++rp) {
       const uint32_t t = byte_pair<B>(WordVec<WPL>::get(q[s][2 * rp + 1], w),
                                       WordVec<WPL>::get(q[s][2 * rp], w));
-      lo[rp] = (t & MASK_LO) | MAGIC_LO;
-      hi[rp] = (t & MASK_HI) | MAGIC_HI;
+      lo[rp] = pk_sub((t & nm.lo) | MAGIC_LO, zl);
+      hi[rp] = pk_sub((t & nm.hi) | MAGIC_HI, zh);
     }
-    const uint32_t zl = zlo[w][B], zh = zhi[w][B];
-    const h8 blo = as_h8(lo) - as_h8(u4v{zl, zl, zl, zl});
-    const h8 bhi = as_h8(hi) - as_h8(u4v{zh, zh, zh, zh});
+    const h8 blo = as_h8(lo);
+    const h8 bhi = as_h8(hi);
     const h8 av = as_h8(a[s]);
     const int t0 = w * 8 + 2 * B;
     const f4 zero = {0.f, 0.f, 0.f, 0.f};
@@ -124,6 +140,16 @@ struct GemvWave {
   }
 
   __device__ __forceinline__ void compute(int s, bool first) {
+#ifdef AWQMI_LAB_NO_COMPUTE    // lab only: consume the loads without the unpack / MFMA work
+    u4v x = a[s];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int w = 0; w < WPL; ++w) x[0] ^= WordVec<WPL>::get(q[s][i], w);
+    accg[0] = __builtin_bit_cast(f4, x);
+    (void)first;
+    return;
+#endif
 #pragma unroll
     for (int w = 0; w < WPL; ++w) {
       tile_pair<0>(s, w, first);
@@ -167,7 +193,11 @@ struct GemvWave {
         build_zdup();
       }
       compute(s, GMODE == 3 ? false : (s % KSPG == 0));
+      // keep the refill of this slot here: sunk to the end of the chunk it would turn the
+      // four-deep load ring into load-all / wait-all / compute-all
+      __builtin_amdgcn_sched_barrier(0);
       if (REFILL) issue(s, c + 1);
+      __builtin_amdgcn_sched_barrier(0);
       if (GMODE < 2 && (s + 1) % KSPG == 0) flush();
     }
     if (GMODE == 2) {
@@ -186,6 +216,7 @@ struct GemvWave {
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
     if (c_begin >= c_end) return;
+    nm.init();
     if (GMODE == 2) load_group(c_begin, zcur, scur);
 #pragma unroll
     for (int s = 0; s < 4; ++s) issue(s, c_begin);
@@ -196,11 +227,11 @@ struct GemvWave {
 };
 
 template <int WPL, int GMODE, bool MOE>
-__global__ __launch_bounds__(256, WPL == 1 ? 2 : 1) void awq_gemv_kernel(const GemvParams p) {
+__global__ __launch_bounds__(256, WPL == 1 ? 3 : 1) void awq_gemv_kernel(const GemvParams p) {
   constexpr int NT = 8 * WPL;
   constexpr int CB = 128 * WPL;
   constexpr int RS = NT * 16 + 4;  // LDS row stride in floats: 4h rows land 16 banks apart
-  __shared__ float red[2][16][RS];
+  __shared__ __align__(16) float red[2][16][RS];
   __shared__ int s_last;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, h = lane >> 4;
@@ -269,24 +300,39 @@ __global__ __launch_bounds__(256, WPL == 1 ? 2 : 1) void awq_gemv_kernel(const G
     // fp32 partial tile of this workgroup, then the arrival counter
     const size_t tile = (size_t)blk * p.ncb + cb;
     const size_t ntiles = (size_t)(MOE ? gridDim.z : 1) * p.ncb;
-    float* mine = p.part + ((size_t)sp * ntiles + tile) * (16 * NT * 16);
-    for (int i = tid; i < nelem; i += 256) {
+    // Partials and the arrival counter go through device-coherent accesses (stores and loads
+    // that bypass the per-XCD L2 for other XCDs' data) instead of full release / acquire
+    // fences: a fence here writes back and invalidates the whole L2 once per workgroup, which
+    // costs far more than the few KB of partials.  Ordering: every store of this workgroup
+    // has completed (vmcnt 0, then the barrier) before its arrival is counted.
+    constexpr int TILE_F = 16 * NT * 16;   // floats per partial tile
+    float* mine = p.part + ((size_t)sp * ntiles + tile) * TILE_F;
+    for (int i = tid * 2; i < nelem; i += 512) {
       const int m = i / (NT * 16), c = i % (NT * 16);
-      mine[i] = red[0][m][c] + red[1][m][c];
+      const f2 v = *reinterpret_cast<const f2*>(&red[0][m][c]) + *reinterpret_cast<const f2*>(&red[1][m][c]);
+      st_coherent(mine + i, v);
     }
-    __threadfence();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) s_last = (atomicAdd(p.cnt + tile, 1) == p.split_k - 1);
     __syncthreads();
     if (!s_last) return;
-    __threadfence();
-    for (int i = tid; i < nelem; i += 256) {
-      float v = 0.f;
-      for (int s = 0; s < p.split_k; ++s)
-        v += __builtin_nontemporal_load(p.part + ((size_t)s * ntiles + tile) * (16 * NT * 16) + i);
-      red[0][i / (NT * 16)][i % (NT * 16)] = v;
+    const float* base = p.part + tile * TILE_F;
+    const size_t sstride = ntiles * TILE_F;
+    for (int i = tid * 2; i < nelem; i += 512) {
+      f2 v = {0.f, 0.f};
+      int s = 0;
+      for (; s + 4 <= p.split_k; s += 4) {   // four independent loads in flight, fixed order
+        const f2 v0 = ld_coherent(base + (size_t)(s + 0) * sstride + i);
+        const f2 v1 = ld_coherent(base + (size_t)(s + 1) * sstride + i);
+        const f2 v2 = ld_coherent(base + (size_t)(s + 2) * sstride + i);
+        const f2 v3 = ld_coherent(base + (size_t)(s + 3) * sstride + i);
+        v = (((v + v0) + v1) + v2) + v3;
+      }
+      for (; s < p.split_k; ++s) v += ld_coherent(base + (size_t)s * sstride + i);
+      *reinterpret_cast<f2*>(&red[0][i / (NT * 16)][i % (NT * 16)]) = v;
     }
-    if (tid == 0) p.cnt[tile] = 0;
+    if (tid == 0) __hip_atomic_store(p.cnt + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
   }
 
