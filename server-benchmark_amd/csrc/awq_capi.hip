@@ -39,11 +39,8 @@ int check_awq_shape(int K, int N, int G) {
   return AWQMI_OK;
 }
 
-// tiled skinny kernel covers: K % 128 == 0 and G in {32, 64, 128 * i}
-inline bool gemv_tiled_ok(int K, int G) {
-  return K % 128 == 0 && (G == 32 || G == 64 || G % 128 == 0);
-}
-inline int gemv_gmode(int G) { return G == 32 ? 0 : (G == 64 ? 1 : (G == 128 ? 2 : 3)); }
+// tiled skinny kernel covers: K a multiple of 128 and G in {32, 64, 128 * i}
+inline bool gemv_tiled_ok(int K, int G) { return K % 128 == 0 && (G == 32 || G == 64 || G % 128 == 0); }
 
 inline int gemv_wpl(int N) {
   const int v = g_gemv_variant.load(std::memory_order_relaxed);
@@ -52,20 +49,30 @@ inline int gemv_wpl(int N) {
 }
 
 // Split-K choice.  The skinny kernel runs one workgroup (one wave per SIMD, 16 KiB of loads
-// in flight per wave) per CU, and that already saturates HBM; a second round of workgroups
-// costs a drain and refill of the memory pipeline.  So: split K just far enough that the
-// launch is a single round of about 256 workgroups, never below one 128-row chunk per wave.
+// in flight per wave) per CU and that saturates HBM; a second round of workgroups costs a
+// drain and refill of the memory pipeline.  So: split K just far enough that the launch is
+// one round of at most 256 workgroups, preferring a split whose 4 x split wave ranges
+// divide the 128-row chunks evenly, never below one chunk per wave.
 int pick_split_k(int rows, int K, int N, int G, long long blocks_z) {
   (void)rows; (void)G;
   const int nchunks = K / 128;
   const long long ncb = (N + 255) / 256;
   const long long wg = ncb * blocks_z;            // workgroups at split 1
-  long long s = (256 + wg / 2) / wg;              // nearest to one workgroup per CU
-  const long long max_split = nchunks / 4 > 0 ? nchunks / 4 : 1;
-  if (s > max_split) s = max_split;
-  if (s > AWQMI_MAX_SPLIT_K) s = AWQMI_MAX_SPLIT_K;
-  if (s < 1) s = 1;
-  return (int)s;
+  long long smax = 256 / wg;                      // largest split that stays within one round
+  if (smax > nchunks / 4) smax = nchunks / 4;
+  if (smax > AWQMI_MAX_SPLIT_K) smax = AWQMI_MAX_SPLIT_K;
+  if (smax < 1) smax = 1;
+  // among splits >= smax / 2 take the one with the best balance (work of the busiest wave)
+  long long best = smax;
+  double best_cost = 1e300;
+  for (long long s = smax; s >= 1 && 2 * s >= smax; --s) {
+    const long long parts = 4 * s;
+    const long long busiest = (nchunks + parts - 1) / parts;
+    const double fill = (double)(wg * s) / 256.0;            // fraction of the round used
+    const double cost = (double)busiest * (double)parts / (double)nchunks / (0.5 + 0.5 * fill);
+    if (cost < best_cost - 1e-9) { best_cost = cost; best = s; }
+  }
+  return (int)best;
 }
 
 inline size_t gemv_partial_bytes(int N, int split, long long blocks_z) {
@@ -75,13 +82,11 @@ inline size_t gemv_partial_bytes(int N, int split, long long blocks_z) {
 }
 
 template <int WPL, bool MOE>
-void launch_gemv(const GemvParams& p, int gmode, dim3 grid, hipStream_t st) {
-  switch (gmode) {
-    case 0: hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MOE>), grid, dim3(256), 0, st, p); break;
-    case 1: hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MOE>), grid, dim3(256), 0, st, p); break;
-    case 2: hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MOE>), grid, dim3(256), 0, st, p); break;
-    default: hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MOE>), grid, dim3(256), 0, st, p); break;
-  }
+void launch_gemv(const GemvParams& p, dim3 grid, hipStream_t st) {
+  if (p.G == 32) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MOE>), grid, dim3(256), 0, st, p);
+  else if (p.G == 64) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MOE>), grid, dim3(256), 0, st, p);
+  else if (p.G == 128) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MOE>), grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MOE>), grid, dim3(256), 0, st, p);
 }
 
 }  // namespace
@@ -187,10 +192,10 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     p.part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
                        : nullptr;
     p.M = M; p.K = K; p.N = N; p.NW = NW; p.G = G;
-    p.nchunks = nchunks; p.cpg = G >= 128 ? G / 128 : 1; p.split_k = split; p.ncb = ncb;
+    p.split_k = split; p.ncb = ncb;
     const dim3 grid(ncb, split, 1);
-    if (wpl == 2) launch_gemv<2, false>(p, gemv_gmode(G), grid, st);
-    else launch_gemv<1, false>(p, gemv_gmode(G), grid, st);
+    if (wpl == 2) launch_gemv<2, false>(p, grid, st);
+    else launch_gemv<1, false>(p, grid, st);
     return launch_status();
   }
 
@@ -305,13 +310,13 @@ int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales
   p.part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
                      : nullptr;
   p.M = 16; p.K = K; p.N = N; p.NW = NW; p.G = G;
-  p.nchunks = nchunks; p.cpg = G >= 128 ? G / 128 : 1; p.split_k = split; p.ncb = ncb;
+  p.split_k = split; p.ncb = ncb;
   p.sorted_ids = sorted_token_ids; p.expert_ids = expert_ids; p.n_post_pad = num_tokens_post_padded;
   p.topk_w = topk_weights; p.n_slots = n_slots; p.a_row_div = a_row_div;
   p.w_stride = (long long)K * NW; p.s_stride = (long long)(K / G) * N; p.z_stride = (long long)(K / G) * NW;
   const dim3 grid(ncb, split, nblk);
-  if (wpl == 2) launch_gemv<2, true>(p, gemv_gmode(G), grid, (hipStream_t)stream);
-  else launch_gemv<1, true>(p, gemv_gmode(G), grid, (hipStream_t)stream);
+  if (wpl == 2) launch_gemv<2, true>(p, grid, (hipStream_t)stream);
+  else launch_gemv<1, true>(p, grid, (hipStream_t)stream);
   return launch_status();
 }
 

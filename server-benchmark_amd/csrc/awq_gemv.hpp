@@ -14,6 +14,10 @@
 #pragma once
 #include "awq_common.hpp"
 
+#ifndef AWQMI_GEMV_WAVES_PER_SIMD
+#define AWQMI_GEMV_WAVES_PER_SIMD 1
+#endif
+
 namespace awqmi {
 
 struct GemvParams {
@@ -25,8 +29,6 @@ struct GemvParams {
   float* part;  // [split][nblk*ncb][16][128*WPL] fp32 partial tiles (tile-major columns)
   int* cnt;     // [nblk*ncb] arrival counters
   int M, K, N, NW, G;
-  int nchunks;  // K / 128
-  int cpg;      // chunks per group when G >= 128
   int split_k;
   int ncb;      // column blocks
   // expert-grouped launch
@@ -64,102 +66,140 @@ struct WordVec<2> {
   static __device__ __forceinline__ uint32_t get(u2v v, int w) { return w ? v.y : v.x; }
 };
 
-// GMODE: 0 -> G = 32, 1 -> G = 64, 2 -> G = 128, 3 -> G = 128 * cpg (cpg > 1)
-template <int WPL, int GMODE, bool MOE>
+// Per-wave main loop.  Ring of four 32-row steps in flight (4 x 8 rows x WPL words + the
+// matching 16-byte activation slice per lane); ring slot = step index mod 4, so a "chunk" is
+// four steps aligned to 128 rows and group boundaries fall on fixed slots.
+//
+// Arithmetic.  A nibble left in place under the mask 0x000F000F (0x00F000F0) *is* the fp16
+// subnormal w * 2^-24 (w * 2^-20), and the matrix core takes subnormal fp16 inputs exactly,
+// so the B operand costs one v_perm_b32 + two v_and_b32 per four weights and no conversion.
+// Per quantisation group and 16-column tile the wave keeps accg = 2^-e * sum_k x_k (w_k - z):
+// the sum over w comes from the unpacked nibbles, the zero point from one more MFMA whose A
+// operand holds this lane's sum of x over the group
+// (split into three fp16 pieces) and whose B operand holds -z * 2^-e.  At the end of the group acc += s * accg (fp32, one
+// v_fma_mix per element); the factor 2^e is applied once when the wave leaves the loop.
+//
+// GMODE: 0 -> G = 32, 1 -> G = 64, 2 -> G = 128, 3 -> G = 128 * i (i > 1).
+template <int WPL, int GMODE>
 struct GemvWave {
-  static constexpr int NT = 8 * WPL;                                    // 16-col tiles / wave
-  static constexpr int KSPG = GMODE == 0 ? 1 : (GMODE == 1 ? 2 : 4);   // 32-row steps / group
+  static constexpr int NT = 8 * WPL;                                   // 16-column tiles per wave
+  static constexpr int KSPG = GMODE == 0 ? 1 : (GMODE == 1 ? 2 : 4);  // group boundaries per chunk
   typedef typename WordVec<WPL>::type qvec;
 
-  const GemvParams& p;
-  const uint32_t* qw;  // lane's column already applied
-  const half_t* sc;
-  const uint32_t* qz;
-  const half_t* xrow;  // lane's activation row, 8h applied
-  int h;
+  const uint32_t* qw_u;  // wave-uniform base of the expert's qweight
+  const half_t* x_lane;  // this lane's activation row, 8h applied
+  uint32_t q_off;        // this lane's byte offset inside a 32-row step: (8h * NW + wc) * 4
+  const half_t* sc;      // lane's scale pointer (8 * wc applied)
+  const uint32_t* qz;    // lane's zero-word pointer (wc applied)
+  int NW, N, kspg, ngroups;   // kspg: 32-row steps per quantisation group
 
   qvec q[4][8];
   u4v a[4];
-  f4 acc[NT];
-  f4 accg[NT];
-  qvec zcur, znext;
-  u4v scur[WPL], snext[WPL];
-  uint32_t zlo[WPL][4], zhi[WPL][4];  // (1024+z, 1024+z) / (64+z, 64+z) per byte of the word
+  f4 acc[NT];    // sum over finished groups of s * accg (still carrying 2^-e)
+  f4 accg[NT];   // current group
+  qvec znext;
+  u4v snext[WPL], scur[WPL];
+  uint32_t zb[NT];   // B operand word of the zero-point MFMA: (-z, -z) * 2^-e
+  float xsum;        // this lane's sum of x over the current group
   NibbleMasks nm;
 
-  __device__ __forceinline__ GemvWave(const GemvParams& pp) : p(pp) {}
-
-  __device__ __forceinline__ void issue(int s, int c) {
-#ifdef AWQMI_LAB_CHUNK_MASK   // lab only: alias all chunks onto a few, so loads hit in L2
-    c &= AWQMI_LAB_CHUNK_MASK;
+  __device__ __forceinline__ void issue(int d, int ks) {
+#ifdef AWQMI_LAB_STEP_MASK   // lab only: alias all steps onto a few, so loads hit in L2
+    ks &= AWQMI_LAB_STEP_MASK;
 #endif
-    const size_t row0 = (size_t)c * 128 + 32 * s + 8 * h;
-    const qvec* src = reinterpret_cast<const qvec*>(qw + row0 * p.NW);
-    const size_t stride = (size_t)p.NW / WPL;
+    const char* rowbase = reinterpret_cast<const char*>(qw_u) + (size_t)ks * 32 * NW * 4;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) q[s][i] = __builtin_nontemporal_load(src + i * stride);
-    a[s] = *reinterpret_cast<const u4v*>(xrow + (size_t)c * 128 + 32 * s);
+    for (int i = 0; i < 8; ++i)
+      q[d][i] = __builtin_nontemporal_load(
+          reinterpret_cast<const qvec*>(rowbase + (size_t)i * NW * 4 + q_off));
+    a[d] = *reinterpret_cast<const u4v*>(x_lane + (size_t)ks * 32);
   }
 
-  __device__ __forceinline__ void load_group(int g, qvec& z, u4v (&s)[WPL]) {
-    z = *reinterpret_cast<const qvec*>(qz + (size_t)g * p.NW);
-#pragma unroll
-    for (int w = 0; w < WPL; ++w) s[w] = *reinterpret_cast<const u4v*>(sc + (size_t)g * p.N + 8 * w);
+  __device__ __forceinline__ int clamp_group(int step) const {
+    const int g = step / kspg;
+    return g < ngroups ? g : ngroups - 1;
   }
 
-  __device__ __forceinline__ void build_zdup() {
+  __device__ __forceinline__ void load_group(int g) {
+    znext = *reinterpret_cast<const qvec*>(qz + (size_t)g * NW);
+#pragma unroll
+    for (int w = 0; w < WPL; ++w) snext[w] = *reinterpret_cast<const u4v*>(sc + (size_t)g * N + 8 * w);
+  }
+
+  // take over the prefetched group parameters
+  __device__ __forceinline__ void adopt_group() {
 #pragma unroll
     for (int w = 0; w < WPL; ++w) {
-      const uint32_t zw = WordVec<WPL>::get(zcur, w);
+      scur[w] = snext[w];
+      const uint32_t zw = WordVec<WPL>::get(znext, w);
       uint32_t t;
-      t = byte_pair<0>(zw, zw); zlo[w][0] = (t & nm.lo) | MAGIC_LO; zhi[w][0] = (t & nm.hi) | MAGIC_HI;
-      t = byte_pair<1>(zw, zw); zlo[w][1] = (t & nm.lo) | MAGIC_LO; zhi[w][1] = (t & nm.hi) | MAGIC_HI;
-      t = byte_pair<2>(zw, zw); zlo[w][2] = (t & nm.lo) | MAGIC_LO; zhi[w][2] = (t & nm.hi) | MAGIC_HI;
-      t = byte_pair<3>(zw, zw); zlo[w][3] = (t & nm.lo) | MAGIC_LO; zhi[w][3] = (t & nm.hi) | MAGIC_HI;
+      t = byte_pair<0>(zw, zw); zb[w * 8 + 0] = (t & nm.lo) | 0x80008000u; zb[w * 8 + 1] = (t & nm.hi) | 0x80008000u;
+      t = byte_pair<1>(zw, zw); zb[w * 8 + 2] = (t & nm.lo) | 0x80008000u; zb[w * 8 + 3] = (t & nm.hi) | 0x80008000u;
+      t = byte_pair<2>(zw, zw); zb[w * 8 + 4] = (t & nm.lo) | 0x80008000u; zb[w * 8 + 5] = (t & nm.hi) | 0x80008000u;
+      t = byte_pair<3>(zw, zw); zb[w * 8 + 6] = (t & nm.lo) | 0x80008000u; zb[w * 8 + 7] = (t & nm.hi) | 0x80008000u;
     }
   }
 
   template <int B>
-  __device__ __forceinline__ void tile_pair(int s, int w, bool first) {
+  __device__ __forceinline__ void tile_pair(int d, int w, bool first) {
     u4v lo, hi;
-    const uint32_t zl = zlo[w][B], zh = zhi[w][B];
 #pragma unroll
     for (int rp = 0; rp < 4; ++rp) {
-      const uint32_t t = byte_pair<B>(WordVec<WPL>::get(q[s][2 * rp + 1], w),
-                                      WordVec<WPL>::get(q[s][2 * rp], w));
-      lo[rp] = pk_sub((t & nm.lo) | MAGIC_LO, zl);
-      hi[rp] = pk_sub((t & nm.hi) | MAGIC_HI, zh);
+      const uint32_t t = byte_pair<B>(WordVec<WPL>::get(q[d][2 * rp + 1], w),
+                                      WordVec<WPL>::get(q[d][2 * rp], w));
+      lo[rp] = t & nm.lo;   // (w_k, w_k+1) * 2^-24 as fp16 subnormals
+      hi[rp] = t & nm.hi;   // (w_k, w_k+1) * 2^-20
     }
-    const h8 blo = as_h8(lo);
-    const h8 bhi = as_h8(hi);
-    const h8 av = as_h8(a[s]);
+    const h8 av = as_h8(a[d]);
     const int t0 = w * 8 + 2 * B;
     const f4 zero = {0.f, 0.f, 0.f, 0.f};
-    accg[t0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, blo, first ? zero : accg[t0], 0, 0, 0);
-    accg[t0 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bhi, first ? zero : accg[t0 + 1], 0, 0, 0);
+    accg[t0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, as_h8(lo), first ? zero : accg[t0], 0, 0, 0);
+    accg[t0 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, as_h8(hi), first ? zero : accg[t0 + 1], 0, 0, 0);
   }
 
-  __device__ __forceinline__ void compute(int s, bool first) {
+  __device__ __forceinline__ void compute(int d, bool first) {
 #ifdef AWQMI_LAB_NO_COMPUTE    // lab only: consume the loads without the unpack / MFMA work
-    u4v x = a[s];
+    u4v x = a[d];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int w = 0; w < WPL; ++w) x[0] ^= WordVec<WPL>::get(q[s][i], w);
-    accg[0] = __builtin_bit_cast(f4, x);
+      for (int w = 0; w < WPL; ++w) x[0] ^= WordVec<WPL>::get(q[d][i], w);
+    acc[0] += __builtin_bit_cast(f4, x);
     (void)first;
     return;
 #endif
+    // this lane's share of sum_k x_k
+    const h2 ones = {(half_t)1.f, (half_t)1.f};
+    float xs = first ? 0.f : xsum;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) xs = __builtin_amdgcn_fdot2(as_h2(a[d][i]), ones, xs, false);
+    xsum = xs;
 #pragma unroll
     for (int w = 0; w < WPL; ++w) {
-      tile_pair<0>(s, w, first);
-      tile_pair<1>(s, w, first);
-      tile_pair<2>(s, w, first);
-      tile_pair<3>(s, w, first);
+      tile_pair<0>(d, w, first);
+      tile_pair<1>(d, w, first);
+      tile_pair<2>(d, w, first);
+      tile_pair<3>(d, w, first);
     }
   }
 
+  // end of a group: zero-point MFMA, then acc += s * accg
   __device__ __forceinline__ void flush() {
+#ifdef AWQMI_LAB_NO_COMPUTE
+    return;
+#endif
+    // xsum as three fp16 pieces (33 significant bits) in k-slots 0..2 against -z in the same slots
+    const half_t x0 = (half_t)xsum;
+    const float r1 = xsum - (float)x0;
+    const half_t x1 = (half_t)r1;
+    const half_t x2 = (half_t)(r1 - (float)x1);
+    const h2 xp01 = {x0, x1}, xp2 = {x2, (half_t)0.f};
+    const h8 az = as_h8(u4v{as_u32(xp01), as_u32(xp2), 0u, 0u});
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const h8 bz = as_h8(u4v{zb[t], zb[t] & 0x0000FFFFu, 0u, 0u});
+      accg[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(az, bz, accg[t], 0, 0, 0);
+    }
 #pragma unroll
     for (int w = 0; w < WPL; ++w) {
       const h8 sv = as_h8(scur[w]);
@@ -172,43 +212,42 @@ struct GemvWave {
     }
   }
 
-  // one 128-row chunk; REFILL: chunk c+1 belongs to this wave too
+  // one aligned 128-row chunk (four ring slots); REFILL: chunk c + 1 belongs to this wave too.
+  // No load sits behind a branch: a branch around a load makes the compiler wait for every
+  // outstanding load at the join, which would empty the ring.
   template <bool REFILL>
   __device__ __forceinline__ void chunk(int c, int c_begin, int c_end) {
-    if (GMODE == 2) {
-      build_zdup();
-      if (REFILL) load_group(c + 1, znext, snext);
-    } else if (GMODE == 3) {
-      if (c == c_begin || c % p.cpg == 0) {
-        load_group(c / p.cpg, zcur, scur);
-        build_zdup();
-#pragma unroll
-        for (int t = 0; t < NT; ++t) accg[t] = f4{0.f, 0.f, 0.f, 0.f};
-      }
+    bool wide_first = false;
+    if (GMODE == 3) {
+      const int cpg = kspg >> 2;
+      wide_first = (c == c_begin) || (c % cpg == 0);
     }
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      if (GMODE < 2 && s % KSPG == 0) {
-        load_group((c * 4 + s) / KSPG, zcur, scur);
-        build_zdup();
+    for (int d = 0; d < 4; ++d) {
+      if (d % KSPG == 0) {
+        adopt_group();
+        if (REFILL || d + KSPG < 4) load_group(clamp_group(4 * c + d + KSPG));
       }
-      compute(s, GMODE == 3 ? false : (s % KSPG == 0));
-      // keep the refill of this slot here: sunk to the end of the chunk it would turn the
-      // four-deep load ring into load-all / wait-all / compute-all
-      __builtin_amdgcn_sched_barrier(0);
-      if (REFILL) issue(s, c + 1);
-      __builtin_amdgcn_sched_barrier(0);
-      if (GMODE < 2 && (s + 1) % KSPG == 0) flush();
-    }
-    if (GMODE == 2) {
-      flush();
-      if (REFILL) {
-        zcur = znext;
+      if (GMODE == 3) {
+        if (d == 0 && wide_first) {
 #pragma unroll
-        for (int w = 0; w < WPL; ++w) scur[w] = snext[w];
+          for (int t = 0; t < NT; ++t) accg[t] = f4{0.f, 0.f, 0.f, 0.f};
+          xsum = 0.f;
+        }
+        compute(d, false);
+      } else {
+        compute(d, d % KSPG == 0);
       }
-    } else if (GMODE == 3) {
-      if (c + 1 == c_end || (c + 1) % p.cpg == 0) flush();
+      // pin the refill right behind its slot's compute: sunk to the end of the chunk the
+      // four-deep ring degenerates into load-all / wait-all / compute-all
+      __builtin_amdgcn_sched_barrier(0);
+      if (REFILL) issue(d, 4 * c + d + 4);
+      __builtin_amdgcn_sched_barrier(0);
+      if (GMODE != 3 && (d + 1) % KSPG == 0) flush();
+    }
+    if (GMODE == 3) {
+      const int cpg = kspg >> 2;
+      if (c + 1 == c_end || (c + 1) % cpg == 0) flush();
     }
   }
 
@@ -217,17 +256,21 @@ struct GemvWave {
     for (int t = 0; t < NT; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
     if (c_begin >= c_end) return;
     nm.init();
-    if (GMODE == 2) load_group(c_begin, zcur, scur);
+    xsum = 0.f;
+    load_group(clamp_group(4 * c_begin));
 #pragma unroll
-    for (int s = 0; s < 4; ++s) issue(s, c_begin);
+    for (int d = 0; d < 4; ++d) issue(d, 4 * c_begin + d);
     int c = c_begin;
     for (; c + 1 < c_end; ++c) chunk<true>(c, c_begin, c_end);
     chunk<false>(c, c_begin, c_end);
+    // undo the 2^-24 / 2^-20 carried by the low- / high-nibble tiles
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] *= (t & 1) ? 1048576.f : 16777216.f;
   }
 };
 
 template <int WPL, int GMODE, bool MOE>
-__global__ __launch_bounds__(256, WPL == 1 ? 3 : 1) void awq_gemv_kernel(const GemvParams p) {
+__global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kernel(const GemvParams p) {
   constexpr int NT = 8 * WPL;
   constexpr int CB = 128 * WPL;
   constexpr int RS = NT * 16 + 4;  // LDS row stride in floats: 4h rows land 16 banks apart
@@ -261,17 +304,25 @@ __global__ __launch_bounds__(256, WPL == 1 ? 3 : 1) void awq_gemv_kernel(const G
     arow = sid < p.n_slots ? (size_t)(sid / p.a_row_div) : 0;
   }
 
-  GemvWave<WPL, GMODE, MOE> w(p);
-  w.qw = qw + wc;
+  GemvWave<WPL, GMODE> w;
+  w.qw_u = qw;
+  w.x_lane = p.x + arow * p.K + 8 * h;
+  w.q_off = (uint32_t)(((size_t)8 * h * p.NW + wc) * 4);
   w.sc = sc + 8 * (size_t)wc;
   w.qz = qz + wc;
-  w.xrow = p.x + arow * p.K + 8 * h;
-  w.h = h;
+  w.NW = p.NW;
+  w.N = p.N;
+  w.kspg = p.G / 32;
+  w.ngroups = p.K / p.G;
 
+  // this wave's share of K, in 128-row chunks; the wave index is made scalar so that the
+  // row base addresses stay in SGPRs
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const long long parts = 4LL * p.split_k;
-  const long long pw = (long long)sp * 4 + wave;
-  const int c_begin = (int)(pw * p.nchunks / parts);
-  const int c_end = (int)((pw + 1) * p.nchunks / parts);
+  const long long pw = (long long)sp * 4 + wave_u;
+  const int nchunks = p.K / 128;
+  const int c_begin = (int)(pw * nchunks / parts);
+  const int c_end = (int)((pw + 1) * nchunks / parts);
   w.run(c_begin, c_end);
 
   // ---- cross-wave sum in LDS: red[b][row][tile*16 + j] ----
