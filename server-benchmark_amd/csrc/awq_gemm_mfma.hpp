@@ -31,13 +31,22 @@ struct MfmaGemmParams {
   int per_xcd;    // ceil(total / 8)
 };
 
-constexpr int PF_BM = 256, PF_BN = 256, PF_BK = 64, PF_LD = 72;
-constexpr int PF_LDS_BYTES = 2 * (PF_BM + PF_BN) * PF_LD * 2;
+constexpr int PF_BM = 256, PF_BN = 256, PF_BK = 64;
+constexpr int PF_ROW_BYTES = PF_BK * 2;                       // 128 B = eight 16-byte slots
+constexpr int PF_TILE_BYTES = PF_BM * PF_ROW_BYTES;           // 32 KiB per operand per buffer
+constexpr int PF_LDS_BYTES = 4 * PF_TILE_BYTES;               // A0 A1 B0 B1
+
+// LDS layout of both operands: [row][64 halves], no padding, the 16-byte slot index XORed
+// with (row ^ (row >> 3)) & 7.  Eight neighbouring rows then put the same logical slot into
+// eight different bank groups (conflict-free fragment reads, lanes = rows), and the eight
+// word columns a wave's neighbouring lanes dequantise (rows 8 apart) do too (conflict-free
+// stores of the dequantised W tile).
+__device__ __forceinline__ int pf_swz(int row) { return (row ^ (row >> 3)) & 7; }
 
 __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmParams p) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  half_t* As = reinterpret_cast<half_t*>(smem_raw);   // [2][256][72]
-  half_t* Bs = As + 2 * PF_BM * PF_LD;                // [2][256][72]
+  unsigned char* const As = smem_raw;                        // [2][256][128 B]
+  unsigned char* const Bs = smem_raw + 2 * PF_TILE_BYTES;    // [2][256][128 B]
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int id = blockIdx.x;
@@ -51,11 +60,35 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   const int m0 = mt_i * PF_BM, n0 = nt_i * PF_BN;
   const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
 
-  // global->LDS roles
-  const int a_row = tid >> 3, a_seg = tid & 7;   // + 32 * i rows
-  const int kk = tid >> 5, wcl = tid & 31;       // 8-row slab, word column in tile
+  // ---- global -> LDS roles -------------------------------------------------------------
+  // X tile: thread (a_row + 32 i, a_seg) moves 16 bytes; rows past M re-read row M - 1 (their
+  // outputs are never stored), so no load sits behind a branch.
+  const int a_row = tid >> 3, a_seg = tid & 7;
+  const half_t* a_src[8];
+  int a_dst[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = a_row + 32 * i;
+    const int gr = min(m0 + r, p.M - 1);
+    a_src[i] = p.x + (size_t)gr * p.K + 8 * a_seg;
+    a_dst[i] = r * PF_ROW_BYTES + ((a_seg ^ pf_swz(r)) << 4);
+  }
+  // W tile: thread (kk, wcl) takes rows 8kk..8kk+7 of word column wcl
+  const int kk = tid >> 5, wcl = tid & 31;
   int wcg = n0 / 8 + wcl;
   if (wcg >= p.NW) wcg = 0;                      // columns never stored; keep loads in bounds
+  const uint32_t* w_src = p.qw + (size_t)8 * kk * p.NW + wcg;
+  const int b_t = kk ^ (wcl & 7);                // slot of column c: (b_t ^ c)
+  const int b_base = wcl * 8 * PF_ROW_BYTES;
+
+  // ---- LDS -> fragment roles -----------------------------------------------------------
+  // lane (i = lane % 32, hh = lane / 32) reads row base + i, logical slot 2 ks + hh; with
+  // u = hh ^ swz(i) the physical slot is u ^ (2 ks) ^ (4 (tile & 1)): four lane offsets
+  const int fi = lane & 31, fh = lane >> 5;
+  const int fu = fh ^ pf_swz(fi);
+  int f_off[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) f_off[c] = fi * PF_ROW_BYTES + ((fu ^ (2 * c)) << 4);
 
   f16v acc[4][4];
 #pragma unroll
@@ -75,20 +108,16 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   auto gload = [&](int kt) {
     const int k0 = kt * PF_BK;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int gr = m0 + a_row + 32 * i;
-      areg[i] = gr < p.M ? *reinterpret_cast<const u4v*>(p.x + (size_t)gr * p.K + k0 + 8 * a_seg)
-                         : u4v{0, 0, 0, 0};
-    }
-    const int kr = k0 + 8 * kk;
+    for (int i = 0; i < 8; ++i) areg[i] = *reinterpret_cast<const u4v*>(a_src[i] + k0);
+    const uint32_t* ws = w_src + (size_t)k0 * p.NW;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) wreg[i] = p.qw[(size_t)(kr + i) * p.NW + wcg];
-    const int g = kr / p.G;
+    for (int i = 0; i < 8; ++i) wreg[i] = ws[(size_t)i * p.NW];
+    const int g = (k0 + 8 * kk) / p.G;
     zreg = p.qz[(size_t)g * p.NW + wcg];
     sreg = *reinterpret_cast<const u4v*>(p.sc + (size_t)g * p.N + 8 * (size_t)wcg);
   };
 
-  auto dq_byte = [&](half_t* bs, auto BTAG) {
+  auto dq_byte = [&](unsigned char* bs, auto BTAG) {
     constexpr int B = decltype(BTAG)::value;
     const uint32_t tz = byte_pair<B>(zreg, zreg);
     const uint32_t zl = (tz & nm.lo) | MAGIC_LO, zh = (tz & nm.hi) | MAGIC_HI;
@@ -106,16 +135,15 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
       lo[rp] = pk_mul(pk_sub((t & nm.lo) | MAGIC_LO, zl), sl);
       hi[rp] = pk_mul(pk_sub((t & nm.hi) | MAGIC_HI, zh), sh);
     }
-    *reinterpret_cast<u4v*>(bs + (8 * wcl + cl) * PF_LD + 8 * kk) = lo;
-    *reinterpret_cast<u4v*>(bs + (8 * wcl + ch) * PF_LD + 8 * kk) = hi;
+    *reinterpret_cast<u4v*>(bs + b_base + cl * PF_ROW_BYTES + ((b_t ^ cl) << 4)) = lo;
+    *reinterpret_cast<u4v*>(bs + b_base + ch * PF_ROW_BYTES + ((b_t ^ ch) << 4)) = hi;
   };
 
   auto sstore = [&](int buf) {
-    half_t* as = As + buf * PF_BM * PF_LD;
-    half_t* bs = Bs + buf * PF_BN * PF_LD;
+    unsigned char* as = As + buf * PF_TILE_BYTES;
+    unsigned char* bs = Bs + buf * PF_TILE_BYTES;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      *reinterpret_cast<u4v*>(as + (a_row + 32 * i) * PF_LD + 8 * a_seg) = areg[i];
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u4v*>(as + a_dst[i]) = areg[i];
     dq_byte(bs, std::integral_constant<int, 0>{});
     dq_byte(bs, std::integral_constant<int, 1>{});
     dq_byte(bs, std::integral_constant<int, 2>{});
@@ -123,15 +151,17 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   };
 
   auto compute = [&](int buf) {
-    const half_t* as = As + buf * PF_BM * PF_LD + (wm + (lane & 31)) * PF_LD + 8 * (lane >> 5);
-    const half_t* bs = Bs + buf * PF_BN * PF_LD + (wn + (lane & 31)) * PF_LD + 8 * (lane >> 5);
+    const unsigned char* as = As + buf * PF_TILE_BYTES + wm * PF_ROW_BYTES;
+    const unsigned char* bs = Bs + buf * PF_TILE_BYTES + wn * PF_ROW_BYTES;
 #pragma unroll
     for (int ks = 0; ks < PF_BK / 16; ++ks) {
       h8 af[4], bf[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const h8*>(as + 32 * i * PF_LD + 16 * ks);
+      for (int i = 0; i < 4; ++i)
+        af[i] = *reinterpret_cast<const h8*>(as + 32 * i * PF_ROW_BYTES + f_off[ks ^ (2 * (i & 1))]);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const h8*>(bs + 32 * j * PF_LD + 16 * ks);
+      for (int j = 0; j < 4; ++j)
+        bf[j] = *reinterpret_cast<const h8*>(bs + 32 * j * PF_ROW_BYTES + f_off[ks ^ (2 * (j & 1))]);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
