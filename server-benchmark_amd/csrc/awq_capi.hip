@@ -199,21 +199,33 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     return launch_status();
   }
 
-  if (M > 16 && K % PF_BK == 0 && G % 8 == 0) {
+  // MFMA kernel: K % 64 == 0, G a power of two >= 8 or a multiple of 64; buffer offsets are
+  // 32-bit, so every operand must stay below 4 GiB
+  const bool pow2g = (G & (G - 1)) == 0 && G >= 8;
+  const bool small = (size_t)M * K * 2 < (1ull << 32) && (size_t)K * NW * 4 < (1ull << 32) &&
+                     (size_t)(K / G) * N * 2 < (1ull << 32);
+  if (M > 16 && K % PF_BK == 0 && (pow2g || G % 64 == 0) && small) {
     static std::atomic<bool> attr_set{false};
     if (!attr_set.load(std::memory_order_acquire)) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(awq_gemm_mfma_kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               PF_LDS_BYTES);
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, PF_LDS_BYTES);
+      if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, PF_LDS_BYTES);
       if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
       attr_set.store(true, std::memory_order_release);
     }
     MfmaGemmParams p{};
     p.x = xx; p.qw = qw; p.sc = sc; p.qz = qz; p.y = yy;
     p.M = M; p.K = K; p.N = N; p.NW = NW; p.G = G;
+    p.gshift = 0;
+    if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
     p.mt = (M + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
     p.total = p.mt * p.nt; p.per_xcd = (p.total + 7) / 8;
-    hipLaunchKernelGGL(awq_gemm_mfma_kernel, dim3(p.per_xcd * 8), dim3(256), PF_LDS_BYTES, st, p);
+    if (pow2g)
+      hipLaunchKernelGGL(awq_gemm_mfma_kernel<true>, dim3(p.per_xcd * 8), dim3(256), PF_LDS_BYTES, st, p);
+    else
+      hipLaunchKernelGGL(awq_gemm_mfma_kernel<false>, dim3(p.per_xcd * 8), dim3(256), PF_LDS_BYTES, st, p);
     return launch_status();
   }
 

@@ -1,16 +1,23 @@
 // Prefill AWQ GEMM (M > 16): Y[M,N] = X[M,K] @ dequant(W) on fp16 MFMA, fp32 accumulate.
 //
 // Workgroup tile 256 x 256 x 64, four waves in a 2 x 2 arrangement, each wave a 128 x 128
-// block of 4 x 4 v_mfma_f32_32x32x16_f16 accumulators (256 accumulator registers).  Both
-// operands sit in LDS k-contiguous ([row][k], row stride 72 halves = 144 B so that eight
-// neighbouring 16-byte reads fall in eight different 16-byte bank groups):
-//   * X tile: 16-byte global loads -> registers -> 16-byte LDS stores;
+// block of 4 x 4 v_mfma_f32_32x32x16_f16 accumulators (256 accumulator registers, one wave
+// per SIMD).  Both operands sit in LDS k-contiguous ([row][64 halves], swizzled, see below):
+//   * X tile: 16-byte buffer loads -> registers -> 16-byte LDS stores;
 //   * W tile: each thread takes 8 rows x 1 packed word (32 threads side by side read 128
 //     contiguous bytes of a row), dequantises its 8 x 8 block to exact fp16 (w - z) * s with
 //     the byte-pair trick (one perm + two and-or per four weights, then packed subtract and
 //     packed multiply), and stores one 16-byte k-run per output column.
-// LDS is double buffered: the global loads of k-tile t+1 are issued before the MFMA loop of
-// tile t, the dequant and LDS stores of t+1 follow it, one barrier per k-tile.
+//
+// Pipeline per k-tile (64 MFMAs per wave = four phases of 16): while tile t is multiplied
+// out of LDS buffer t & 1, tile t + 1 goes from registers into the other buffer (X stores in
+// phase 1, W dequantisation spread over phases 1-3, each interleaved between the MFMAs) and
+// tile t + 2 is fetched from global memory into the freed registers.  The workgroup barrier
+// sits between phase 3 and phase 4: phase 4 multiplies fragments that are already in
+// registers, so behind the barrier it overlaps the first fragment reads of tile t + 1.
+// Global addresses are buffer loads with a loop-invariant lane offset and a scalar offset
+// that advances per tile, so the loop carries no vector address arithmetic.
+//
 // Workgroup ids are spread over the eight XCDs in contiguous ranges and walked in
 // 8-row-tile groups so that the 32 workgroups resident on one XCD share X and W tiles
 // through that XCD's L2.
@@ -26,6 +33,7 @@ struct MfmaGemmParams {
   const uint32_t* qz;
   half_t* y;
   int M, K, N, NW, G;
+  int gshift;     // log2(G) when G is a power of two (kernel instantiation POW2G)
   int mt, nt;     // tile counts
   int total;      // mt * nt
   int per_xcd;    // ceil(total / 8)
@@ -43,6 +51,14 @@ constexpr int PF_LDS_BYTES = 4 * PF_TILE_BYTES;               // A0 A1 B0 B1
 // stores of the dequantised W tile).
 __device__ __forceinline__ int pf_swz(int row) { return (row ^ (row >> 3)) & 7; }
 
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* base, size_t bytes) {
+  const uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
+}
+
+// POW2G: G is a power of two (group index by shift, any G >= 8); otherwise G % 64 == 0 and
+// a k-tile lies inside one group (group index on the scalar unit).
+template <bool POW2G>
 __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmParams p) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   unsigned char* const As = smem_raw;                        // [2][256][128 B]
@@ -60,10 +76,14 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   const int m0 = mt_i * PF_BM, n0 = nt_i * PF_BN;
   const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
 
+  const __amdgpu_buffer_rsrc_t rx = pf_rsrc(p.x, (size_t)p.M * p.K * 2);
+  const __amdgpu_buffer_rsrc_t rw = pf_rsrc(p.qw, (size_t)p.K * p.NW * 4);
+  const __amdgpu_buffer_rsrc_t rz = pf_rsrc(p.qz, (size_t)(p.K / p.G) * p.NW * 4);
+  const __amdgpu_buffer_rsrc_t rs = pf_rsrc(p.sc, (size_t)(p.K / p.G) * p.N * 2);
+
   // ---- global -> LDS roles -------------------------------------------------------------
   // X tile: thread (a_row + 32 i, a_seg) moves 16 bytes; rows past M re-read row M - 1 (their
-  // outputs are never stored), so no load sits behind a branch.  Addresses are a uniform
-  // base (advanced per k-tile on the scalar unit) plus a 32-bit lane offset.
+  // outputs are never stored), so no load sits behind a branch.
   const int a_row = tid >> 3, a_seg = tid & 7;
   uint32_t a_off[8];
   int a_dst[8];
@@ -79,8 +99,8 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   int wcg = n0 / 8 + wcl;
   if (wcg >= p.NW) wcg = 0;                      // columns never stored; keep loads in bounds
   const uint32_t w_off = (uint32_t)(((size_t)8 * kk * p.NW + wcg) * 4);
-  const uint32_t w_row = (uint32_t)p.NW * 4;     // bytes between rows
-  const int b_t = kk ^ (wcl & 7);                // slot of column c: (b_t ^ c)
+  const uint32_t row_b = (uint32_t)p.NW * 4;     // bytes between qweight / qzeros rows
+  const int b_t = kk ^ (wcl & 7);                // physical slot of column c: b_t ^ c
   const int b_base = wcl * 8 * PF_ROW_BYTES;
 
   // ---- LDS -> fragment roles -----------------------------------------------------------
@@ -109,18 +129,24 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   const int KT = p.K / PF_BK;
 
   auto gload_a = [&](int kt) {
-    const char* base = reinterpret_cast<const char*>(p.x) + (size_t)kt * PF_BK * 2;
+    const int so = kt * (PF_BK * 2);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) areg[i] = *reinterpret_cast<const u4v*>(base + a_off[i]);
+    for (int i = 0; i < 8; ++i) areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, a_off[i], so, 0);
   };
   auto gload_w = [&](int kt, int set) {
-    const char* base = reinterpret_cast<const char*>(p.qw) + (size_t)kt * PF_BK * p.NW * 4;
+    const uint32_t so = (uint32_t)kt * PF_BK * row_b;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      wreg[set][i] = *reinterpret_cast<const uint32_t*>(base + (size_t)i * w_row + w_off);
-    const int g = (kt * PF_BK + 8 * kk) / p.G;
-    zreg[set] = p.qz[(size_t)g * p.NW + wcg];
-    sreg[set] = *reinterpret_cast<const u4v*>(p.sc + (size_t)g * p.N + 8 * (size_t)wcg);
+      wreg[set][i] = __builtin_amdgcn_raw_buffer_load_b32(rw, w_off, so + i * row_b, 0);
+    if (POW2G) {
+      const uint32_t g = (uint32_t)(kt * PF_BK + 8 * kk) >> p.gshift;
+      zreg[set] = __builtin_amdgcn_raw_buffer_load_b32(rz, g * row_b + wcg * 4, 0, 0);
+      sreg[set] = __builtin_amdgcn_raw_buffer_load_b128(rs, (g * (uint32_t)p.N + 8 * wcg) * 2, 0, 0);
+    } else {
+      const uint32_t g = (uint32_t)(kt * PF_BK) / (uint32_t)p.G;
+      zreg[set] = __builtin_amdgcn_raw_buffer_load_b32(rz, wcg * 4, g * row_b, 0);
+      sreg[set] = __builtin_amdgcn_raw_buffer_load_b128(rs, wcg * 16, g * (uint32_t)p.N * 2, 0);
+    }
   };
   auto store_a = [&](int buf) {
     unsigned char* as = As + buf * PF_TILE_BYTES;
@@ -169,79 +195,92 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[fs][i], bf[fs][j], acc[i][j], 0, 0, 0);
   };
 
-  // Interleave recipe for one phase (16 MFMAs of one 16-wide k-step, the eight fragment
-  // reads of the next one, the dequantisation of one byte of the next W tile): an MFMA
-  // occupies the matrix pipe for eight passes, during which the wave can issue about seven
-  // other instructions, so spread the VALU / LDS work evenly between the MFMAs.
-  auto phase_schedule = [&](bool with_reads) {
+  // Interleave recipe for one phase of 16 MFMAs: an MFMA occupies the matrix pipe for eight
+  // passes, during which the wave can issue about seven other instructions, so the other
+  // work of the phase is dealt out evenly between the MFMAs: per MFMA pair `valu` VALU ops,
+  // `dsr` LDS reads, `dsw` LDS writes and `vm` buffer loads.
+  auto phase_schedule = [&](auto VALU, auto DSR, auto DSW, auto VM) {
+    constexpr int valu = decltype(VALU)::value, dsr = decltype(DSR)::value;
+    constexpr int dsw = decltype(DSW)::value, vm = decltype(VM)::value;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // MFMA
-      if (with_reads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);               // VALU
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);               // VALU
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (dsr) __builtin_amdgcn_sched_group_barrier(0x100, dsr, 0);
+      if (vm) __builtin_amdgcn_sched_group_barrier(0x020, vm, 0);
+      if (valu) __builtin_amdgcn_sched_group_barrier(0x002, (valu + 1) / 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (dsw) __builtin_amdgcn_sched_group_barrier(0x200, dsw, 0);
+      if (valu / 2) __builtin_amdgcn_sched_group_barrier(0x002, valu / 2, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);                 // DS write
   };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+  using I6 = std::integral_constant<int, 6>;
+  using I12 = std::integral_constant<int, 12>;
 
-  // One k-tile, PAR = kt & 1.  On entry: LDS buffer PAR holds tile kt, areg and W set PAR^1
-  // hold tile kt + 1, W set PAR is free.  The body stores X(kt+1), refills areg and W set
-  // PAR with tile kt + 2, then runs the four 16-wide k-steps of tile kt: each step's MFMAs
-  // overlap the fragment reads of the next step and one byte of the dequantisation of
-  // W(kt+1).  Tiles past the end re-read the last tile and are never used.
+  // One k-tile, PAR = kt & 1.  On entry: LDS buffer PAR holds tile kt and fragment set 0 its
+  // first k-step; areg and W set PAR^1 hold tile kt + 1; W set PAR is free.  Tiles past the
+  // end re-read the last tile and are never used.
   auto body = [&](int kt, auto PTAG) {
     constexpr int PAR = decltype(PTAG)::value;
     const int kt2 = min(kt + 2, KT - 1);
-    store_a(PAR ^ 1);
-    __builtin_amdgcn_sched_barrier(0);
-    gload_a(kt2);
-    gload_w(kt2, PAR);
-    load_frags(PAR, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
 
+    // phase 1: X(kt+1) -> LDS, W(kt+2) -> registers, byte 0 of W(kt+1)
     mfma_step(0);
     load_frags(PAR, 1, 1);
-    dq_byte(PAR ^ 1, PAR ^ 1, std::integral_constant<int, 0>{});
-    phase_schedule(true);
+    store_a(PAR ^ 1);
+    gload_w(kt2, PAR);
+    dq_byte(PAR ^ 1, PAR ^ 1, I0{});
+    phase_schedule(I6{}, I1{}, I1{}, I2{});
     __builtin_amdgcn_sched_barrier(0);
 
+    // phase 2: X(kt+2) -> registers, byte 1 of W(kt+1)
     mfma_step(1);
     load_frags(PAR, 2, 0);
-    dq_byte(PAR ^ 1, PAR ^ 1, std::integral_constant<int, 1>{});
-    phase_schedule(true);
+    gload_a(kt2);
+    dq_byte(PAR ^ 1, PAR ^ 1, I1{});
+    phase_schedule(I6{}, I1{}, I1{}, I1{});
     __builtin_amdgcn_sched_barrier(0);
 
+    // phase 3: bytes 2 and 3 of W(kt+1)
     mfma_step(0);
     load_frags(PAR, 3, 1);
-    dq_byte(PAR ^ 1, PAR ^ 1, std::integral_constant<int, 2>{});
-    phase_schedule(true);
+    dq_byte(PAR ^ 1, PAR ^ 1, I2{});
+    dq_byte(PAR ^ 1, PAR ^ 1, I3{});
+    phase_schedule(I12{}, I1{}, I1{}, I0{});
     __builtin_amdgcn_sched_barrier(0);
 
-    mfma_step(1);
-    dq_byte(PAR ^ 1, PAR ^ 1, std::integral_constant<int, 3>{});
-    phase_schedule(false);
-    __builtin_amdgcn_sched_barrier(0);
+    // every LDS write of tile kt + 1 is out and every read of tile kt has returned
     __syncthreads();
+
+    // phase 4: last k-step from registers, first fragments of tile kt + 1
+    mfma_step(1);
+    load_frags(PAR ^ 1, 0, 0);
+    phase_schedule(I0{}, I1{}, I0{}, I0{});
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   // prologue: tile 0 into LDS buffer 0, tile 1 into registers
   gload_a(0);
   gload_w(0, 0);
   store_a(0);
-  dq_byte(0, 0, std::integral_constant<int, 0>{});
-  dq_byte(0, 0, std::integral_constant<int, 1>{});
-  dq_byte(0, 0, std::integral_constant<int, 2>{});
-  dq_byte(0, 0, std::integral_constant<int, 3>{});
+  dq_byte(0, 0, I0{});
+  dq_byte(0, 0, I1{});
+  dq_byte(0, 0, I2{});
+  dq_byte(0, 0, I3{});
   gload_a(min(1, KT - 1));
   gload_w(min(1, KT - 1), 1);
   __syncthreads();
+  load_frags(0, 0, 0);
+  __builtin_amdgcn_sched_barrier(0);
   int kt = 0;
   for (; kt + 1 < KT; kt += 2) {
-    body(kt, std::integral_constant<int, 0>{});
-    body(kt + 1, std::integral_constant<int, 1>{});
+    body(kt, I0{});
+    body(kt + 1, I1{});
   }
-  if (kt < KT) body(kt, std::integral_constant<int, 0>{});
+  if (kt < KT) body(kt, I0{});
 
   // D[i][j] of a 32x32 tile: j = lane % 32, i = 8 * (r / 4) + 4 * (lane / 32) + r % 4
   const int col_l = lane & 31, row_l = 4 * (lane >> 5);
