@@ -29,6 +29,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
+# HBM bytes per awq_gemv launch averaged over the decode sweep, from two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE) of `bench.py --pmc-target decode`, each scaled by what the same
+# counter reads for a 256 MiB device copy; the runs are summarised in
+# profiles/awq_gemv_kernel_decode_sweep_pmc_hbm_traffic.md.  Counters cannot be read while
+# timing, so the figure is carried here and is only valid for the default split-K choice.
+DECODE_SWEEP_TRAFFIC_BYTES = 118946302
 
 
 def log(*a):
@@ -56,6 +62,13 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--detail", action="store_true", help="per-point timings on stderr")
+    ap.add_argument("--sweep-only", action="store_true",
+                    help="only the timed decode sweep (no per-point, prefill, dequantize, MoE or CPU legs)")
+    ap.add_argument("--pmc-target", choices=("decode", "prefill"), default=None,
+                    help="counter-collection mode for rocprofv3 --pmc, no timing.  decode: the 16-launch "
+                         "decode sweep twice (direct launches) plus four 256 MiB device copies "
+                         "(calibration of FETCH_SIZE / WRITE_SIZE).  prefill: awq_gemm at o_proj, "
+                         "M=8192, three times")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -111,6 +124,34 @@ def main():
     step_bytes = sum(workloads.linear_bytes(M, K, N, G) for _, K, N in layers for M in Ms)
     n_launch = len(layers) * len(Ms)
 
+    if args.pmc_target == "prefill":
+        name, K, N = layers[1]
+        qw, sc, qz = W[name][0]
+        xp = torch.randn((8192, K), device=dev, generator=gen).to(torch.float16)
+        yp = torch.empty((8192, N), dtype=torch.float16, device=dev)
+        for _ in range(3):
+            st = lib.awqmi_gemm_f16(xp.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), yp.data_ptr(),
+                                    ws.data_ptr(), ws.numel(), 8192, K, N, G, 0,
+                                    torch.cuda.current_stream().cuda_stream)
+            assert st == 0
+        torch.cuda.synchronize()
+        log(f"[bench] pmc target: 3 x awq_gemm {name} M=8192 K={K} N={N} "
+            f"({workloads.linear_flops(8192, K, N)} flops each)")
+        return
+    if args.pmc_target == "decode":
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        sp = torch.cuda.current_stream().cuda_stream
+        step(sp)
+        step(sp)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        log(f"[bench] pmc target: 2 decode sweeps = {2 * n_launch} awq_gemm launches, "
+            f"{step_bytes / n_launch:.0f} algorithmic bytes per launch on average; "
+            f"4 device copies of {src.numel()} bytes")
+        return
+
     graph = None
     if args.launch == "graph":
         side = torch.cuda.Stream()
@@ -148,11 +189,13 @@ def main():
     log(f"[bench] decode sweep: {ms_per_step:.3f} ms/step wall, {ev_ms / args.steps:.3f} ms/step events, "
         f"{value:.0f} GB/s ({value / HBM_PEAK_GBS:.1%} of {HBM_PEAK_GBS:.0f})")
 
+    if args.sweep_only:
+        args.no_prefill = args.no_cpu = True
     # per-point detail (direct launches, event pair per point, same rotation)
     points = []
     stream_ptr = torch.cuda.current_stream().cuda_stream
     reps = 10
-    for name, K, N in layers:
+    for name, K, N in ([] if args.sweep_only else layers):
         for ci, M in enumerate(Ms):
             # flush the last-level cache with the other layers' copies between points
             evs = []
@@ -195,7 +238,9 @@ def main():
                                "16 awq_gemm launches per step, 4 rotating weight copies per layer",
                    "launch": args.launch, "split_k": args.split_k, "bytes_per_step": step_bytes},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": DECODE_SWEEP_TRAFFIC_BYTES if args.split_k == 0 and args.variant < 0 else None,
+                     "traffic_source": "profiles/awq_gemv_kernel_decode_sweep_pmc_hbm_traffic.md",
                      "kernel": "awq_gemv_kernel", "avg_launch_us": round(kern_avg_us, 2),
                      "bytes_per_launch": step_bytes // n_launch},
         "decode_points": points,
@@ -242,6 +287,72 @@ def main():
                           "frac": round(agg / MFMA_FP16_PEAK_TFLOPS, 4), "kernel": "awq_gemm_mfma_kernel",
                           "points": pts}
         log(f"[bench] prefill sweep aggregate {agg:.1f} TFLOP/s ({agg / MFMA_FP16_PEAK_TFLOPS:.1%} of fp16 MFMA peak)")
+
+    # ------------------------------------------------------------------ awq_dequantize (write-bound)
+    if not args.no_prefill:
+        dq = []
+        for name, K, N in layers:
+            qw, sc, qz = W[name][0]
+            o = torch.empty((K, N), dtype=torch.float16, device=dev)
+
+            def call():
+                st = lib.awqmi_dequantize_f16(qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), o.data_ptr(), K, N, G,
+                                              stream_ptr)
+                if st != 0:
+                    raise RuntimeError(lib.awqmi_status_string(st).decode())
+
+            call()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(5):
+                call()
+            b.record()
+            torch.cuda.synchronize()
+            us = a.elapsed_time(b) * 1e3 / 5
+            nbytes = workloads.linear_bytes(0, K, N, G) + 2 * K * N     # packed in + fp16 out
+            dq.append({"layer": name, "K": K, "N": N, "us": round(us, 1), "GBps": round(nbytes / us / 1e3, 1),
+                       "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+            del o
+        out["dequantize"] = {"unit": "GB/s", "kernel": "awq_dequant_kernel", "bound": "hbm (write)", "points": dq}
+
+    # ------------------------------------------------------------------ fused MoE block (Qwen3-30B-A3B shapes)
+    if not args.no_prefill:
+        mq = workloads.QWEN3_MOE
+        H, E, topk, I = mq["hidden"], mq["experts"], mq["topk"], mq["inter"]
+        w13 = [make_weights(H, 2 * I, G, dev, gen) for _ in range(E)]
+        w2 = [make_weights(I, H, G, dev, gen) for _ in range(E)]
+        w13 = tuple(torch.stack([w[i] for w in w13]) for i in range(3))
+        w2 = tuple(torch.stack([w[i] for w in w2]) for i in range(3))
+        mo = []
+        for T in workloads.MOE_T:
+            xm = torch.randn((T, H), device=dev, generator=gen).to(torch.float16)
+            lg = torch.randn((T, E), device=dev, generator=gen)
+            for _ in range(3):
+                ym = sba.fused_moe_awq(xm, w13, w2, lg, topk, True)
+            torch.cuda.synchronize()
+            _, ids = sba.topk_softmax(lg, topk, True)
+            distinct = int(torch.unique(ids).numel())
+            n_it = 20
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(n_it):
+                ym = sba.fused_moe_awq(xm, w13, w2, lg, topk, True)
+            b.record()
+            torch.cuda.synchronize()
+            us = a.elapsed_time(b) * 1e3 / n_it
+            nbytes = workloads.moe_bytes(distinct, T, H, I, G)
+            fl = workloads.moe_flops(T, topk, H, I)
+            mo.append({"T": T, "distinct_experts": distinct, "us": round(us, 1),
+                       "GBps": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                       "TFLOPs": round(fl / us / 1e6, 2)})
+            if args.detail:
+                log(f"   moe T={T:4d} experts hit {distinct:3d}  {us:9.1f} us  {nbytes / us / 1e3:8.1f} GB/s")
+        out["moe"] = {"workload": "Qwen3-30B-A3B MoE block: route + align + grouped w13 GEMM + SiLU*up + grouped w2 "
+                                  "GEMM + slot sum, 128 experts, top-8, hidden 2048, inter 768 (whole block per call, "
+                                  "weights not rotated: cache-warm for small T)",
+                      "points": mo}
+        del w13, w2
 
     # ------------------------------------------------------------------ CPU baseline leg
     if not args.no_cpu:
