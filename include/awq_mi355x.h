@@ -40,7 +40,7 @@ typedef enum awqmi_status {
 } awqmi_status;
 
 #define AWQMI_VERSION 100        /* major*10000 + minor*100 + patch */
-#define AWQMI_MOE_TILE_M 16      /* rows per sorted-token block the grouped GEMM consumes  */
+#define AWQMI_MOE_TILE_M 16      /* default rows per sorted-token block (32 also accepted)  */
 #define AWQMI_MAX_SPLIT_K 64
 #define AWQMI_MAX_EXPERTS 1024
 
@@ -71,8 +71,8 @@ size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k);
  * Stands in for vLLM's `awq_gemm` op (every AWQ Linear at decode and prefill); reached
  * from the server started at reference utils/generate_compose.py:85-93.
  * fp32 accumulation, one final rounding to fp16.  M >= 1; K % group == 0; N % 8 == 0.
- * M <= 16 takes the HBM-bound skinny kernel (split_k honoured, 0 = auto), larger M the
- * LDS-dequant MFMA kernel (split_k ignored).  Shapes outside the fast kernels' tiling
+ * M <= 64 takes the HBM-bound skinny kernel in passes of up to 32 rows (split_k honoured,
+ * 0 = auto), larger M the LDS-dequant MFMA kernel (split_k ignored).  Shapes outside the fast kernels' tiling
  * (K % 128 != 0, group not in {32, 64, 128*i}) take a slow generic kernel. */
 int awqmi_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
                    const int32_t* qzeros, void* y_f16, void* workspace, size_t workspace_bytes,
@@ -98,9 +98,11 @@ int awqmi_moe_align(const int32_t* topk_ids, int n_slots, int E, int tile_m,
                     int32_t* num_tokens_post_padded, void* stream);
 
 /* Workspace bytes of one grouped GEMM call (same counter rule as awqmi_gemm_f16). */
-size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int split_k);
+size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int split_k, int tile_m);
 
-/* Expert-grouped AWQ GEMM over sorted-token blocks of AWQMI_MOE_TILE_M rows.
+/* Expert-grouped AWQ GEMM over sorted-token blocks of tile_m rows (16, or 32 when the
+ * average expert load makes 16-row blocks re-read weights; the ids must come from
+ * awqmi_moe_align with the same tile_m).
  * For every non-pad entry s = sorted_token_ids[i] in a block owned by expert e:
  *     y[s, :] = (x[s / a_row_div, :] @ W_e) * (topk_weights ? topk_weights[s] : 1)
  * a_row_div = topk for the first GEMM (x is [T, K]), 1 for the second (x is [n_slots, K]).
@@ -110,8 +112,8 @@ size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int spli
 int awqmi_moe_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
                        const int32_t* qzeros, void* y_f16, const int32_t* sorted_token_ids,
                        const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
-                       const float* topk_weights, int n_slots, int a_row_div, int E, int K, int N,
-                       int group, int split_k, void* workspace, size_t workspace_bytes,
+                       const float* topk_weights, int n_slots, int a_row_div, int tile_m, int E, int K,
+                       int N, int group, int split_k, void* workspace, size_t workspace_bytes,
                        void* stream);
 
 /* out[r, i] = silu(in[r, i]) * in[r, inter + i], in fp16 [rows, 2*inter] ([gate | up]),

@@ -75,19 +75,22 @@ int pick_split_k(int rows, int K, int N, int G, long long blocks_z) {
   return (int)best;
 }
 
-inline size_t gemv_partial_bytes(int N, int split, long long blocks_z) {
+inline size_t gemv_partial_bytes(int N, int split, long long blocks_z, int tile_m = 16) {
   if (split <= 1) return 0;
   const size_t npad = ((size_t)N + 255) / 256 * 256;
-  return (size_t)split * (size_t)blocks_z * 16 * npad * sizeof(float);
+  return (size_t)split * (size_t)blocks_z * tile_m * npad * sizeof(float);
 }
 
-template <int WPL, bool MOE>
+template <int WPL, int MB, bool MOE>
 void launch_gemv(const GemvParams& p, dim3 grid, hipStream_t st) {
-  if (p.G == 32) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MOE>), grid, dim3(256), 0, st, p);
-  else if (p.G == 64) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MOE>), grid, dim3(256), 0, st, p);
-  else if (p.G == 128) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MOE>), grid, dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MOE>), grid, dim3(256), 0, st, p);
+  if (p.G == 32) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MB, MOE>), grid, dim3(256), 0, st, p);
+  else if (p.G == 64) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MB, MOE>), grid, dim3(256), 0, st, p);
+  else if (p.G == 128) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MB, MOE>), grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MB, MOE>), grid, dim3(256), 0, st, p);
 }
+
+// rows the skinny kernel takes in one awq_gemm call (passes of up to 32 rows)
+constexpr int SKINNY_MAX_M = 64;
 
 }  // namespace
 
@@ -142,16 +145,16 @@ int awqmi_dequantize_f16(const int32_t* qweight, const void* scales, const int32
 int awqmi_gemm_auto_split_k(int M, int K, int N, int group) {
   const int G = norm_group(K, group);
   if (check_awq_shape(K, N, G) != AWQMI_OK || M <= 0) return 1;
-  if (M > 16 || !gemv_tiled_ok(K, G)) return 1;
+  if (M > SKINNY_MAX_M || !gemv_tiled_ok(K, G)) return 1;
   return pick_split_k(M, K, N, G, 1);
 }
 
 size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
   if (M <= 0 || K <= 0 || N <= 0) return 0;
-  if (M > 16) return AWQMI_WS_COUNTER_BYTES;
+  if (M > SKINNY_MAX_M) return AWQMI_WS_COUNTER_BYTES;
   int s = split_k;
   if (s <= 0) s = (K % 128 == 0) ? pick_split_k(M, K, N, 128, 1) : 1;
-  return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, s, 1);
+  return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, s, 1, 32);
 }
 
 int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
@@ -173,29 +176,36 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   const half_t* xx = reinterpret_cast<const half_t*>(x);
   half_t* yy = reinterpret_cast<half_t*>(y);
 
-  if (M <= 16 && gemv_tiled_ok(K, G)) {
+  const int wpl = gemv_wpl(N);
+  if (gemv_tiled_ok(K, G) && (M <= 16 || (M <= SKINNY_MAX_M && wpl == 2))) {
     int split = split_k > 0 ? split_k : pick_split_k(M, K, N, G, 1);
     const int nchunks = K / 128;
     if (split > nchunks) split = nchunks;
-    const int wpl = gemv_wpl(N);
     const int ncb = (NW + 16 * wpl - 1) / (16 * wpl);
     if (split > 1) {
       if (!workspace) return AWQMI_NULL_POINTER;
       if (!aligned16(workspace)) return AWQMI_BAD_ALIGN;
       if ((size_t)ncb * sizeof(int) > AWQMI_WS_COUNTER_BYTES) return AWQMI_BAD_SHAPE;
-      if (workspace_bytes < AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, split, 1))
+      if (workspace_bytes < AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, split, 1, M > 16 ? 32 : 16))
         return AWQMI_WORKSPACE_TOO_SMALL;
     }
     GemvParams p{};
-    p.x = xx; p.qw = qw; p.sc = sc; p.qz = qz; p.y = yy;
+    p.qw = qw; p.sc = sc; p.qz = qz;
     p.cnt = reinterpret_cast<int*>(workspace);
     p.part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
                        : nullptr;
-    p.M = M; p.K = K; p.N = N; p.NW = NW; p.G = G;
+    p.K = K; p.N = N; p.NW = NW; p.G = G;
     p.split_k = split; p.ncb = ncb;
     const dim3 grid(ncb, split, 1);
-    if (wpl == 2) launch_gemv<2, false>(p, grid, st);
-    else launch_gemv<1, false>(p, grid, st);
+    // passes of up to 32 rows; each pass streams the weights once
+    for (int r0 = 0; r0 < M; r0 += 32) {
+      p.x = xx + (size_t)r0 * K;
+      p.y = yy + (size_t)r0 * N;
+      p.M = M - r0 < 32 ? M - r0 : 32;
+      if (p.M > 16) launch_gemv<2, 2, false>(p, grid, st);
+      else if (wpl == 2) launch_gemv<2, 1, false>(p, grid, st);
+      else launch_gemv<1, 1, false>(p, grid, st);
+    }
     return launch_status();
   }
 
@@ -204,7 +214,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   const bool pow2g = (G & (G - 1)) == 0 && G >= 8;
   const bool small = (size_t)M * K * 2 < (1ull << 32) && (size_t)K * NW * 4 < (1ull << 32) &&
                      (size_t)(K / G) * N * 2 < (1ull << 32);
-  if (M > 16 && K % PF_BK == 0 && (pow2g || G % 64 == 0) && small) {
+  if (K % PF_BK == 0 && (pow2g || G % 64 == 0) && small) {
     static std::atomic<bool> attr_set{false};
     if (!attr_set.load(std::memory_order_acquire)) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true>),
@@ -263,9 +273,9 @@ int awqmi_moe_align(const int32_t* topk_ids, int n_slots, int E, int tile_m, int
   return launch_status();
 }
 
-static int moe_pick_split(int n_slots, int E, int K, int N, int G, int nblk, int ncb) {
-  // blocks that will actually run: at most one per 16 slots plus one per expert touched
-  long long live = (n_slots + 15) / 16;
+static int moe_pick_split(int n_slots, int E, int K, int N, int G, int nblk, int ncb, int tile_m) {
+  // blocks that will actually run: at most one per tile_m slots plus one per expert touched
+  long long live = (n_slots + tile_m - 1) / tile_m;
   const long long touched = n_slots < E ? n_slots : E;
   if (live < touched) live = touched;
   int s = pick_split_k(16, K, N, G, live);
@@ -273,26 +283,27 @@ static int moe_pick_split(int n_slots, int E, int K, int N, int G, int nblk, int
   return s;
 }
 
-size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int split_k) {
-  if (n_slots <= 0 || E <= 0 || K <= 0 || N <= 0) return 0;
-  const int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, AWQMI_MOE_TILE_M) / AWQMI_MOE_TILE_M);
+size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int split_k, int tile_m) {
+  if (n_slots <= 0 || E <= 0 || K <= 0 || N <= 0 || (tile_m != 16 && tile_m != 32)) return 0;
+  const int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, tile_m) / tile_m);
   int s = split_k;
-  if (s <= 0) s = (K % 128 == 0) ? moe_pick_split(n_slots, E, K, N, 128, nblk, (N + 127) / 128) : 1;
-  return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, s, nblk);
+  if (s <= 0) s = (K % 128 == 0) ? moe_pick_split(n_slots, E, K, N, 128, nblk, (N + 127) / 128, tile_m) : 1;
+  return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, s, nblk, tile_m);
 }
 
 int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
                        void* y, const int32_t* sorted_token_ids, const int32_t* expert_ids,
                        const int32_t* num_tokens_post_padded, const float* topk_weights, int n_slots,
-                       int a_row_div, int E, int K, int N, int group, int split_k, void* workspace,
-                       size_t workspace_bytes, void* stream) {
+                       int a_row_div, int tile_m, int E, int K, int N, int group, int split_k,
+                       void* workspace, size_t workspace_bytes, void* stream) {
   if (!x || !qweight || !scales || !qzeros || !y || !sorted_token_ids || !expert_ids ||
       !num_tokens_post_padded)
     return AWQMI_NULL_POINTER;
   const int G = norm_group(K, group);
   if (int st = check_awq_shape(K, N, G)) return st;
   if (n_slots <= 0 || E <= 0) return AWQMI_BAD_SHAPE;
-  if (a_row_div <= 0 || split_k < 0 || split_k > AWQMI_MAX_SPLIT_K || E > AWQMI_MAX_EXPERTS)
+  if (a_row_div <= 0 || split_k < 0 || split_k > AWQMI_MAX_SPLIT_K || E > AWQMI_MAX_EXPERTS ||
+      (tile_m != 16 && tile_m != 32))
     return AWQMI_BAD_ARGUMENT;
   if (!gemv_tiled_ok(K, G)) return AWQMI_UNSUPPORTED_GROUP;
   if (!aligned16(x) || !aligned16(scales) || !aligned16(qweight) || !aligned16(qzeros) ||
@@ -300,16 +311,17 @@ int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales
     return AWQMI_BAD_ALIGN;
   const int NW = N / 8;
   const int wpl = gemv_wpl(N);
+  if (tile_m == 32 && wpl != 2) return AWQMI_BAD_SHAPE;   // 32-row blocks need N % 16 == 0
   const int ncb = (NW + 16 * wpl - 1) / (16 * wpl);
-  const int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, AWQMI_MOE_TILE_M) / AWQMI_MOE_TILE_M);
-  int split = split_k > 0 ? split_k : moe_pick_split(n_slots, E, K, N, G, nblk, ncb);
+  const int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, tile_m) / tile_m);
+  int split = split_k > 0 ? split_k : moe_pick_split(n_slots, E, K, N, G, nblk, ncb, tile_m);
   const int nchunks = K / 128;
   if (split > nchunks) split = nchunks;
   if (split > 1) {
     if (!workspace) return AWQMI_NULL_POINTER;
     if (!aligned16(workspace)) return AWQMI_BAD_ALIGN;
     if ((size_t)nblk * ncb * sizeof(int) > AWQMI_WS_COUNTER_BYTES) return AWQMI_BAD_ARGUMENT;
-    if (workspace_bytes < AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, split, nblk))
+    if (workspace_bytes < AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, split, nblk, tile_m))
       return AWQMI_WORKSPACE_TOO_SMALL;
   }
   GemvParams p{};
@@ -321,14 +333,16 @@ int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales
   p.cnt = reinterpret_cast<int*>(workspace);
   p.part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
                      : nullptr;
-  p.M = 16; p.K = K; p.N = N; p.NW = NW; p.G = G;
+  p.M = tile_m; p.K = K; p.N = N; p.NW = NW; p.G = G;
   p.split_k = split; p.ncb = ncb;
   p.sorted_ids = sorted_token_ids; p.expert_ids = expert_ids; p.n_post_pad = num_tokens_post_padded;
-  p.topk_w = topk_weights; p.n_slots = n_slots; p.a_row_div = a_row_div;
+  p.topk_w = topk_weights; p.n_slots = n_slots; p.a_row_div = a_row_div; p.tile_m = tile_m;
   p.w_stride = (long long)K * NW; p.s_stride = (long long)(K / G) * N; p.z_stride = (long long)(K / G) * NW;
   const dim3 grid(ncb, split, nblk);
-  if (wpl == 2) launch_gemv<2, true>(p, grid, (hipStream_t)stream);
-  else launch_gemv<1, true>(p, grid, (hipStream_t)stream);
+  hipStream_t st = (hipStream_t)stream;
+  if (tile_m == 32) launch_gemv<2, 2, true>(p, grid, st);
+  else if (wpl == 2) launch_gemv<2, 1, true>(p, grid, st);
+  else launch_gemv<1, 1, true>(p, grid, st);
   return launch_status();
 }
 

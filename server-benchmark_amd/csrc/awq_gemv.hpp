@@ -38,6 +38,7 @@ struct GemvParams {
   const float* topk_w;
   int n_slots;
   int a_row_div;
+  int tile_m;   // rows per sorted-token block: 16 * MB
   long long w_stride, s_stride, z_stride;  // elements per expert
 };
 
@@ -67,7 +68,7 @@ struct WordVec<2> {
 };
 
 // Per-wave main loop.  Ring of four 32-row steps in flight (4 x 8 rows x WPL words + the
-// matching 16-byte activation slice per lane); ring slot = step index mod 4, so a "chunk" is
+// matching 16-byte activation slices per lane); ring slot = step index mod 4, so a "chunk" is
 // four steps aligned to 128 rows and group boundaries fall on fixed slots.
 //
 // Arithmetic.  A nibble left in place under the mask 0x000F000F (0x00F000F0) *is* the fp16
@@ -75,32 +76,33 @@ struct WordVec<2> {
 // so the B operand costs one v_perm_b32 + two v_and_b32 per four weights and no conversion.
 // Per quantisation group and 16-column tile the wave keeps accg = 2^-e * sum_k x_k (w_k - z):
 // the sum over w comes from the unpacked nibbles, the zero point from one more MFMA whose A
-// operand holds this lane's sum of x over the group
-// (split into three fp16 pieces) and whose B operand holds -z * 2^-e.  At the end of the group acc += s * accg (fp32, one
-// v_fma_mix per element); the factor 2^e is applied once when the wave leaves the loop.
+// operand holds this lane's sum of x over the group (split into three fp16 pieces) and whose
+// B operand holds -z * 2^-e.  At the end of the group acc += s * accg (fp32, one v_fma_mix per
+// element); the factor 2^e is applied once when the wave leaves the loop.
 //
-// GMODE: 0 -> G = 32, 1 -> G = 64, 2 -> G = 128, 3 -> G = 128 * i (i > 1).
-template <int WPL, int GMODE>
+// MB row blocks of 16 share every B operand (MB = 2 serves up to 32 rows per pass with the
+// unpack work of one).  GMODE: 0 -> G = 32, 1 -> G = 64, 2 -> G = 128, 3 -> G = 128 * i.
+template <int WPL, int GMODE, int MB>
 struct GemvWave {
   static constexpr int NT = 8 * WPL;                                   // 16-column tiles per wave
   static constexpr int KSPG = GMODE == 0 ? 1 : (GMODE == 1 ? 2 : 4);  // group boundaries per chunk
   typedef typename WordVec<WPL>::type qvec;
 
-  const uint32_t* qw_u;  // wave-uniform base of the expert's qweight
-  const half_t* x_lane;  // this lane's activation row, 8h applied
-  uint32_t q_off;        // this lane's byte offset inside a 32-row step: (8h * NW + wc) * 4
-  const half_t* sc;      // lane's scale pointer (8 * wc applied)
-  const uint32_t* qz;    // lane's zero-word pointer (wc applied)
-  int NW, N, kspg, ngroups;   // kspg: 32-row steps per quantisation group
+  const uint32_t* qw_u;      // wave-uniform base of the expert's qweight
+  const half_t* x_lane[MB];  // this lane's activation row per row block, 8h applied
+  uint32_t q_off;            // this lane's byte offset inside a 32-row step: (8h * NW + wc) * 4
+  const half_t* sc;          // lane's scale pointer (8 * wc applied)
+  const uint32_t* qz;        // lane's zero-word pointer (wc applied)
+  int NW, N, kspg, ngroups;  // kspg: 32-row steps per quantisation group
 
   qvec q[4][8];
-  u4v a[4];
-  f4 acc[NT];    // sum over finished groups of s * accg (still carrying 2^-e)
-  f4 accg[NT];   // current group
+  u4v a[4][MB];
+  f4 acc[MB][NT];    // sum over finished groups of s * accg (still carrying 2^-e)
+  f4 accg[MB][NT];   // current group
   qvec znext;
   u4v snext[WPL], scur[WPL];
   uint32_t zb[NT];   // B operand word of the zero-point MFMA: (-z, -z) * 2^-e
-  float xsum;        // this lane's sum of x over the current group
+  float xsum[MB];    // this lane's sum of x over the current group
   NibbleMasks nm;
 
   __device__ __forceinline__ void issue(int d, int ks) {
@@ -112,7 +114,9 @@ struct GemvWave {
     for (int i = 0; i < 8; ++i)
       q[d][i] = __builtin_nontemporal_load(
           reinterpret_cast<const qvec*>(rowbase + (size_t)i * NW * 4 + q_off));
-    a[d] = *reinterpret_cast<const u4v*>(x_lane + (size_t)ks * 32);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      a[d][mb] = *reinterpret_cast<const u4v*>(x_lane[mb] + (size_t)ks * 32);
   }
 
   __device__ __forceinline__ int clamp_group(int step) const {
@@ -150,30 +154,37 @@ struct GemvWave {
       lo[rp] = t & nm.lo;   // (w_k, w_k+1) * 2^-24 as fp16 subnormals
       hi[rp] = t & nm.hi;   // (w_k, w_k+1) * 2^-20
     }
-    const h8 av = as_h8(a[d]);
     const int t0 = w * 8 + 2 * B;
     const f4 zero = {0.f, 0.f, 0.f, 0.f};
-    accg[t0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, as_h8(lo), first ? zero : accg[t0], 0, 0, 0);
-    accg[t0 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, as_h8(hi), first ? zero : accg[t0 + 1], 0, 0, 0);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const h8 av = as_h8(a[d][mb]);
+      accg[mb][t0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, as_h8(lo), first ? zero : accg[mb][t0], 0, 0, 0);
+      accg[mb][t0 + 1] =
+          __builtin_amdgcn_mfma_f32_16x16x32_f16(av, as_h8(hi), first ? zero : accg[mb][t0 + 1], 0, 0, 0);
+    }
   }
 
   __device__ __forceinline__ void compute(int d, bool first) {
 #ifdef AWQMI_LAB_NO_COMPUTE    // lab only: consume the loads without the unpack / MFMA work
-    u4v x = a[d];
+    u4v x = a[d][0];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
       for (int w = 0; w < WPL; ++w) x[0] ^= WordVec<WPL>::get(q[d][i], w);
-    acc[0] += __builtin_bit_cast(f4, x);
+    acc[0][0] += __builtin_bit_cast(f4, x);
     (void)first;
     return;
 #endif
     // this lane's share of sum_k x_k
     const h2 ones = {(half_t)1.f, (half_t)1.f};
-    float xs = first ? 0.f : xsum;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) xs = __builtin_amdgcn_fdot2(as_h2(a[d][i]), ones, xs, false);
-    xsum = xs;
+    for (int mb = 0; mb < MB; ++mb) {
+      float xs = first ? 0.f : xsum[mb];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) xs = __builtin_amdgcn_fdot2(as_h2(a[d][mb][i]), ones, xs, false);
+      xsum[mb] = xs;
+    }
 #pragma unroll
     for (int w = 0; w < WPL; ++w) {
       tile_pair<0>(d, w, first);
@@ -188,26 +199,29 @@ struct GemvWave {
 #ifdef AWQMI_LAB_NO_COMPUTE
     return;
 #endif
-    // xsum as three fp16 pieces (33 significant bits) in k-slots 0..2 against -z in the same slots
-    const half_t x0 = (half_t)xsum;
-    const float r1 = xsum - (float)x0;
-    const half_t x1 = (half_t)r1;
-    const half_t x2 = (half_t)(r1 - (float)x1);
-    const h2 xp01 = {x0, x1}, xp2 = {x2, (half_t)0.f};
-    const h8 az = as_h8(u4v{as_u32(xp01), as_u32(xp2), 0u, 0u});
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const h8 bz = as_h8(u4v{zb[t], zb[t] & 0x0000FFFFu, 0u, 0u});
-      accg[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(az, bz, accg[t], 0, 0, 0);
-    }
+    for (int mb = 0; mb < MB; ++mb) {
+      // xsum as three fp16 pieces (33 significant bits) in k-slots 0..2 against -z there
+      const half_t x0 = (half_t)xsum[mb];
+      const float r1 = xsum[mb] - (float)x0;
+      const half_t x1 = (half_t)r1;
+      const half_t x2 = (half_t)(r1 - (float)x1);
+      const h2 xp01 = {x0, x1}, xp2 = {x2, (half_t)0.f};
+      const h8 az = as_h8(u4v{as_u32(xp01), as_u32(xp2), 0u, 0u});
 #pragma unroll
-    for (int w = 0; w < WPL; ++w) {
-      const h8 sv = as_h8(scur[w]);
+      for (int t = 0; t < NT; ++t) {
+        const h8 bz = as_h8(u4v{zb[t], zb[t] & 0x0000FFFFu, 0u, 0u});
+        accg[mb][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(az, bz, accg[mb][t], 0, 0, 0);
+      }
 #pragma unroll
-      for (int nib = 0; nib < 8; ++nib) {
-        const float s = (float)sv[awq_col_of_nibble(nib)];
-        const int t = w * 8 + nib;
-        acc[t] += s * accg[t];
+      for (int w = 0; w < WPL; ++w) {
+        const h8 sv = as_h8(scur[w]);
+#pragma unroll
+        for (int nib = 0; nib < 8; ++nib) {
+          const float s = (float)sv[awq_col_of_nibble(nib)];
+          const int t = w * 8 + nib;
+          acc[mb][t] += s * accg[mb][t];
+        }
       }
     }
   }
@@ -231,8 +245,11 @@ struct GemvWave {
       if (GMODE == 3) {
         if (d == 0 && wide_first) {
 #pragma unroll
-          for (int t = 0; t < NT; ++t) accg[t] = f4{0.f, 0.f, 0.f, 0.f};
-          xsum = 0.f;
+          for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) accg[mb][t] = f4{0.f, 0.f, 0.f, 0.f};
+            xsum[mb] = 0.f;
+          }
         }
         compute(d, false);
       } else {
@@ -253,10 +270,13 @@ struct GemvWave {
 
   __device__ __forceinline__ void run(int c_begin, int c_end) {
 #pragma unroll
-    for (int t = 0; t < NT; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
+    for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[mb][t] = f4{0.f, 0.f, 0.f, 0.f};
+      xsum[mb] = 0.f;
+    }
     if (c_begin >= c_end) return;
     nm.init();
-    xsum = 0.f;
     load_group(clamp_group(4 * c_begin));
 #pragma unroll
     for (int d = 0; d < 4; ++d) issue(d, 4 * c_begin + d);
@@ -265,15 +285,18 @@ struct GemvWave {
     chunk<false>(c, c_begin, c_end);
     // undo the 2^-24 / 2^-20 carried by the low- / high-nibble tiles
 #pragma unroll
-    for (int t = 0; t < NT; ++t) acc[t] *= (t & 1) ? 1048576.f : 16777216.f;
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[mb][t] *= (t & 1) ? 1048576.f : 16777216.f;
   }
 };
 
-template <int WPL, int GMODE, bool MOE>
+template <int WPL, int GMODE, int MB, bool MOE>
 __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kernel(const GemvParams p) {
   constexpr int NT = 8 * WPL;
   constexpr int CB = 128 * WPL;
   constexpr int RS = NT * 16 + 4;  // LDS row stride in floats: 4h rows land 16 banks apart
+  constexpr int TM = 16 * MB;      // rows per pass
   __shared__ __align__(16) float red[2][16][RS];
   __shared__ int s_last;
 
@@ -285,7 +308,7 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
   const uint32_t* qz = p.qz;
   if (MOE) {
     blk = blockIdx.z;
-    if (blk * 16 >= *p.n_post_pad) return;
+    if (blk * TM >= *p.n_post_pad) return;
     const int e = p.expert_ids[blk];
     qw += (size_t)e * p.w_stride;
     sc += (size_t)e * p.s_stride;
@@ -296,17 +319,21 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
   // / row 0 instead; their B column (resp. A row) only feeds outputs that are never stored.
   int wc = cb * (16 * WPL) + WPL * j;
   if (wc >= p.NW) wc = 0;
-  size_t arow;
-  if (!MOE) {
-    arow = j < p.M ? (size_t)j : 0;
-  } else {
-    const int sid = p.sorted_ids[blk * 16 + j];
-    arow = sid < p.n_slots ? (size_t)(sid / p.a_row_div) : 0;
-  }
 
-  GemvWave<WPL, GMODE> w;
+  GemvWave<WPL, GMODE, MB> w;
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int r = mb * 16 + j;
+    size_t arow;
+    if (!MOE) {
+      arow = r < p.M ? (size_t)r : 0;
+    } else {
+      const int sid = p.sorted_ids[blk * TM + r];
+      arow = sid < p.n_slots ? (size_t)(sid / p.a_row_div) : 0;
+    }
+    w.x_lane[mb] = p.x + arow * p.K + 8 * h;
+  }
   w.qw_u = qw;
-  w.x_lane = p.x + arow * p.K + 8 * h;
   w.q_off = (uint32_t)(((size_t)8 * h * p.NW + wc) * 4);
   w.sc = sc + 8 * (size_t)wc;
   w.qz = qz + wc;
@@ -325,89 +352,107 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
   const int c_end = (int)((pw + 1) * nchunks / parts);
   w.run(c_begin, c_end);
 
-  // ---- cross-wave sum in LDS: red[b][row][tile*16 + j] ----
-  if (wave >= 2) {
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) red[wave - 2][4 * h + r][t * 16 + j] = w.acc[t][r];
-  }
-  __syncthreads();
-  if (wave < 2) {
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) red[wave][4 * h + r][t * 16 + j] += w.acc[t][r];
-  }
-  __syncthreads();
-
-  int rows = p.M;
+  int rows_total = p.M;
   if (MOE) {  // valid slots sit at the front of a block, pads behind them
-    rows = 0;
-    for (int m = 0; m < 16; ++m) rows += p.sorted_ids[blk * 16 + m] < p.n_slots ? 1 : 0;
+    rows_total = 0;
+    for (int m = 0; m < TM; ++m) rows_total += p.sorted_ids[blk * TM + m] < p.n_slots ? 1 : 0;
   }
-  const int nelem = rows * (NT * 16);
-  if (p.split_k > 1) {
-    // fp32 partial tile of this workgroup, then the arrival counter
-    const size_t tile = (size_t)blk * p.ncb + cb;
-    const size_t ntiles = (size_t)(MOE ? gridDim.z : 1) * p.ncb;
-    // Partials and the arrival counter go through device-coherent accesses (stores and loads
-    // that bypass the per-XCD L2 for other XCDs' data) instead of full release / acquire
-    // fences: a fence here writes back and invalidates the whole L2 once per workgroup, which
-    // costs far more than the few KB of partials.  Ordering: every store of this workgroup
-    // has completed (vmcnt 0, then the barrier) before its arrival is counted.
-    constexpr int TILE_F = 16 * NT * 16;   // floats per partial tile
-    float* mine = p.part + ((size_t)sp * ntiles + tile) * TILE_F;
-    for (int i = tid * 2; i < nelem; i += 512) {
-      const int m = i / (NT * 16), c = i % (NT * 16);
-      const f2 v = *reinterpret_cast<const f2*>(&red[0][m][c]) + *reinterpret_cast<const f2*>(&red[1][m][c]);
-      st_coherent(mine + i, v);
+  const size_t tile = (size_t)blk * p.ncb + cb;
+  const size_t ntiles = (size_t)(MOE ? gridDim.z : 1) * p.ncb;
+  constexpr int TILE_F = 16 * NT * 16;   // floats per partial tile (one row block)
+  const bool split = p.split_k > 1;
+
+  // tile-major LDS (red[0], optionally + red[1]) -> row-major fp16 output of row block mb
+  auto emit = [&](int mb, int rows, bool two) {
+    for (int i = tid; i < rows * CB; i += 256) {
+      const int m = i / CB, cl = i % CB;
+      const int wl = cl >> 3;                 // word within the block
+      const int jj = wl / WPL, ww = wl % WPL;
+      const int t = ww * 8 + awq_nibble_of_col(cl & 7);
+      const int col = cb * CB + cl;
+      float v = red[0][m][t * 16 + jj];
+      if (two) v += red[1][m][t * 16 + jj];
+      if (col >= p.N) continue;
+      if (!MOE) {
+        p.y[(size_t)(mb * 16 + m) * p.N + col] = (half_t)v;
+      } else {
+        const int sid = p.sorted_ids[blk * TM + mb * 16 + m];
+        if (sid < p.n_slots) {
+          if (p.topk_w) v *= p.topk_w[sid];
+          p.y[(size_t)sid * p.N + col] = (half_t)v;
+        }
+      }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  };
+
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int rows = min(16, max(0, rows_total - 16 * mb));
+    // ---- cross-wave sum in LDS: red[b][row][tile*16 + j] ----
+    if (wave >= 2) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[wave - 2][4 * h + r][t * 16 + j] = w.acc[mb][t][r];
+    }
     __syncthreads();
-    if (tid == 0) s_last = (atomicAdd(p.cnt + tile, 1) == p.split_k - 1);
+    if (wave < 2) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[wave][4 * h + r][t * 16 + j] += w.acc[mb][t][r];
+    }
     __syncthreads();
-    if (!s_last) return;
-    const float* base = p.part + tile * TILE_F;
-    const size_t sstride = ntiles * TILE_F;
+    if (split) {
+      // fp32 partial tile of this workgroup.  Partials and the arrival counter go through
+      // device-coherent accesses (they bypass the per-XCD L2 for other XCDs' data) instead of
+      // release / acquire fences: a fence here writes back and invalidates the whole L2 once
+      // per workgroup, which costs far more than the few KB of partials.
+      float* mine = p.part + (((size_t)sp * ntiles + tile) * MB + mb) * TILE_F;
+      const int nelem = rows * (NT * 16);
+      for (int i = tid * 2; i < nelem; i += 512) {
+        const int m = i / (NT * 16), c = i % (NT * 16);
+        const f2 v = *reinterpret_cast<const f2*>(&red[0][m][c]) + *reinterpret_cast<const f2*>(&red[1][m][c]);
+        st_coherent(mine + i, v);
+      }
+    } else {
+      emit(mb, rows, true);
+    }
+    __syncthreads();
+  }
+  if (!split) return;
+
+  // Ordering: every store of this workgroup has completed (vmcnt 0, then the barrier)
+  // before its arrival is counted; whoever arrives last sums all partials in fixed order.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (tid == 0) s_last = (atomicAdd(p.cnt + tile, 1) == p.split_k - 1);
+  __syncthreads();
+  if (!s_last) return;
+  const size_t sstride = ntiles * MB * TILE_F;
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int rows = min(16, max(0, rows_total - 16 * mb));
+    const int nelem = rows * (NT * 16);
+    const float* base = p.part + (tile * MB + mb) * TILE_F;
     for (int i = tid * 2; i < nelem; i += 512) {
       f2 v = {0.f, 0.f};
       int s = 0;
-      for (; s + 4 <= p.split_k; s += 4) {   // four independent loads in flight, fixed order
-        const f2 v0 = ld_coherent(base + (size_t)(s + 0) * sstride + i);
-        const f2 v1 = ld_coherent(base + (size_t)(s + 1) * sstride + i);
-        const f2 v2 = ld_coherent(base + (size_t)(s + 2) * sstride + i);
-        const f2 v3 = ld_coherent(base + (size_t)(s + 3) * sstride + i);
-        v = (((v + v0) + v1) + v2) + v3;
+      for (; s + 8 <= p.split_k; s += 8) {   // eight independent loads in flight, fixed order
+        f2 t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) t[u] = ld_coherent(base + (size_t)(s + u) * sstride + i);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v += t[u];
       }
       for (; s < p.split_k; ++s) v += ld_coherent(base + (size_t)s * sstride + i);
       *reinterpret_cast<f2*>(&red[0][i / (NT * 16)][i % (NT * 16)]) = v;
     }
-    if (tid == 0) __hip_atomic_store(p.cnt + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    emit(mb, rows, false);
     __syncthreads();
   }
-
-  // ---- tile-major LDS -> row-major fp16 output ----
-  const bool summed = p.split_k > 1;
-  for (int i = tid; i < rows * CB; i += 256) {
-    const int m = i / CB, cl = i % CB;
-    const int wl = cl >> 3;                 // word within the block
-    const int jj = wl / WPL, ww = wl % WPL;
-    const int t = ww * 8 + awq_nibble_of_col(cl & 7);
-    const int col = cb * CB + cl;
-    float v = red[0][m][t * 16 + jj];
-    if (!summed) v += red[1][m][t * 16 + jj];
-    if (col >= p.N) continue;
-    if (!MOE) {
-      p.y[(size_t)m * p.N + col] = (half_t)v;
-    } else {
-      const int sid = p.sorted_ids[blk * 16 + m];
-      if (sid < p.n_slots) {
-        if (p.topk_w) v *= p.topk_w[sid];
-        p.y[(size_t)sid * p.N + col] = (half_t)v;
-      }
-    }
-  }
+  if (tid == 0) __hip_atomic_store(p.cnt + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace awqmi

@@ -150,9 +150,10 @@ def moe_awq_gemm(a: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, q
                  sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
                  num_tokens_post_padded: torch.Tensor, n_slots: int, a_row_div: int,
                  topk_weights: torch.Tensor | None = None, split_k: int = 0,
-                 out: torch.Tensor | None = None) -> torch.Tensor:
-    """Expert-grouped AWQ GEMM over blocks of 16 sorted slots: out[s] = a[s // a_row_div] @
-    W[expert(s)] (* topk_weights[s])."""
+                 out: torch.Tensor | None = None, block_size: int = MOE_TILE_M) -> torch.Tensor:
+    """Expert-grouped AWQ GEMM over blocks of `block_size` (16 or 32) sorted slots:
+    out[s] = a[s // a_row_div] @ W[expert(s)] (* topk_weights[s]).  The ids must come from
+    moe_align_block_size with the same block size."""
     _need(a, "a", torch.float16, 2)
     _need(qweight, "qweight", torch.int32, 3)
     _need(scales, "scales", torch.float16, 3)
@@ -167,8 +168,10 @@ def moe_awq_gemm(a: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, q
     if a.shape[0] * a_row_div < n_slots:
         raise ValueError("a has too few rows for n_slots / a_row_div")
     lib = _lib.load()
-    cap = lib.awqmi_moe_align_capacity(n_slots, E, MOE_TILE_M)
-    if sorted_token_ids.numel() < cap or expert_ids.numel() < cap // MOE_TILE_M:
+    if block_size not in (16, 32):
+        raise ValueError("block_size must be 16 or 32")
+    cap = lib.awqmi_moe_align_capacity(n_slots, E, block_size)
+    if sorted_token_ids.numel() < cap or expert_ids.numel() < cap // block_size:
         raise ValueError("sorted_token_ids / expert_ids smaller than the align capacity")
     tw = 0
     if topk_weights is not None:
@@ -179,12 +182,12 @@ def moe_awq_gemm(a: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, q
     if out is None:
         out = torch.empty((n_slots, N), dtype=torch.float16, device=a.device)
     split = max(0, min(int(split_k), 64))
-    nbytes = lib.awqmi_moe_gemm_workspace_bytes(n_slots, E, K, N, split)
+    nbytes = lib.awqmi_moe_gemm_workspace_bytes(n_slots, E, K, N, split, block_size)
     ws = get_workspace(a.device, nbytes)
     st = lib.awqmi_moe_gemm_f16(a.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
                                 out.data_ptr(), sorted_token_ids.data_ptr(), expert_ids.data_ptr(),
-                                num_tokens_post_padded.data_ptr(), tw, n_slots, a_row_div, E, K, N, G,
-                                split, ws.data_ptr(), ws.numel(), _stream_ptr(a.device))
+                                num_tokens_post_padded.data_ptr(), tw, n_slots, a_row_div, block_size, E, K,
+                                N, G, split, ws.data_ptr(), ws.numel(), _stream_ptr(a.device))
     _lib.check(st, "moe_awq_gemm")
     return out
 
@@ -218,9 +221,12 @@ def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Ten
     T = hidden_states.shape[0]
     E = w13[0].shape[0]
     topk_w, topk_ids = topk_softmax(gating_output.float().contiguous(), topk, renormalize)
-    sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, MOE_TILE_M, E)
     n = T * topk
-    h13 = moe_awq_gemm(hidden_states, *w13, sorted_ids, expert_ids, npp, n, topk)
+    # 32-row blocks once an expert sees more than ~16 slots on average: one pass over its
+    # weights instead of two
+    bs = 32 if n > 16 * E else MOE_TILE_M
+    sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, bs, E)
+    h13 = moe_awq_gemm(hidden_states, *w13, sorted_ids, expert_ids, npp, n, topk, block_size=bs)
     act = silu_and_mul(h13)
-    o = moe_awq_gemm(act, *w2, sorted_ids, expert_ids, npp, n, 1, topk_weights=topk_w)
+    o = moe_awq_gemm(act, *w2, sorted_ids, expert_ids, npp, n, 1, topk_weights=topk_w, block_size=bs)
     return moe_sum(o, T, topk)

@@ -65,6 +65,32 @@ def test_moe_fixture(sba, gpu):
     assert err <= TOL
 
 
+@pytest.mark.parametrize("bs", [16, 32])
+def test_moe_grouped_gemm_block_sizes(sba, gpu, bs):
+    """The grouped GEMM alone, 16- and 32-row blocks, against per-slot oracle products."""
+    rng = np.random.default_rng(40 + bs)
+    T, E, topk, K, N, G = 37, 8, 2, 256, 264 if bs == 16 else 256, 128
+    w = rng.integers(0, 16, (E, K, N))
+    z = rng.integers(0, 16, (E, K // G, N))
+    s = (rng.random((E, K // G, N)) * 0.019 + 0.001).astype(np.float16)
+    qw, qz = awq_ref.pack_awq(w), awq_ref.pack_awq(z)
+    x = rng.normal(0, 1, (T, K)).astype(np.float16)
+    ids = np.stack([rng.choice(E, size=topk, replace=False) for _ in range(T)]).astype(np.int32)
+    tw = rng.random((T, topk)).astype(np.float32)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+    sid, eid, npp = sba.moe_align_block_size(t(ids), bs, E)
+    y = sba.moe_awq_gemm(t(x), t(qw), t(s), t(qz), sid, eid, npp, T * topk, topk, topk_weights=t(tw),
+                         split_k=2, block_size=bs).cpu().numpy()
+    ref = np.zeros((T * topk, N))
+    for tok in range(T):
+        for slot in range(topk):
+            e = ids[tok, slot]
+            ref[tok * topk + slot] = awq_ref.gemm_wide(x[tok:tok + 1], qw[e], s[e], qz[e], G)[0] * tw[tok, slot]
+    err = awq_ref.rel_frobenius(y, ref)
+    print(f"[moe grouped gemm bs={bs}] rel_fro={err:.2e}", flush=True)
+    assert err <= TOL
+
+
 @pytest.mark.parametrize("T", [1, 16])
 def test_moe_qwen3_shapes_vs_oracle(sba, gpu, T):
     c = sba.workloads.make_moe_case(T, 2048, 128, 8, 768, 128, seed=100 + T)

@@ -109,6 +109,17 @@ def test_gemm_decode_groups_and_ragged_n(sba, gpu, K, N, G):
         _check_gemm(sba, gpu, x, qw, s, qz, g, split)
 
 
+@pytest.mark.parametrize("M", [17, 24, 32, 33, 48, 64])
+def test_gemm_mid_m_skinny_passes(sba, gpu, M):
+    """17 <= M <= 64 runs the skinny kernel in passes of up to 32 rows (two row blocks share
+    every unpacked weight)."""
+    x, qw, s, qz = _np_case(M, 1024, 512, 128, seed=200 + M)
+    for split in (0, 1, 4):
+        _check_gemm(sba, gpu, x, qw, s, qz, 128, split, tag="mid-M")
+    x, qw, s, qz = _np_case(M, 512, 264, 64, seed=300 + M)      # ragged N, G = 64
+    _check_gemm(sba, gpu, x, qw, s, qz, 64, 0, tag="mid-M")
+
+
 def test_gemm_one_hot_is_exact_and_zero_weights(sba, gpu):
     K, N, G = 512, 256, 128
     _, qw, s, qz = _np_case(1, K, N, G, seed=77)
@@ -131,8 +142,8 @@ def test_gemm_one_hot_is_exact_and_zero_weights(sba, gpu):
     bound = np.abs(xr.astype(np.float64)).sum(axis=1, keepdims=True) * 15 * float(s.max()) * 2.0 ** -18
     print(f"[w == z] max |y| = {np.abs(y).max():.3e}, bound {bound.min():.3e}", flush=True)
     assert np.all(np.abs(y.astype(np.float64)) <= bound)
-    # the MFMA path (M > 16) dequantises to exact fp16 zeros first: exact zeros there
-    xl = np.random.default_rng(1).normal(0, 1, (40, K)).astype(np.float16)
+    # the MFMA path (M > 64) dequantises to exact fp16 zeros first: exact zeros there
+    xl = np.random.default_rng(1).normal(0, 1, (80, K)).astype(np.float16)
     assert not sba.awq_gemm(*_dev(gpu, xl, awq_ref.pack_awq(zfull), s, qz), 0).cpu().numpy().any()
 
 

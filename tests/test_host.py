@@ -59,8 +59,10 @@ def test_validation_happens_before_any_launch(lib):
     assert lib.awqmi_moe_align(0, 8, 4, 16, fake, fake, fake, 0) == 6
     assert lib.awqmi_moe_align(fake, 8, 2000, 16, fake, fake, fake, 0) == 7
     assert lib.awqmi_moe_topk_softmax_f32(fake, 4, 8, 9, 1, fake, fake, 0) == 7
-    assert lib.awqmi_moe_gemm_f16(fake, fake, fake, fake, fake, fake, fake, fake, 0, 8, 2, 4, 100, 64, 50,
+    assert lib.awqmi_moe_gemm_f16(fake, fake, fake, fake, fake, fake, fake, fake, 0, 8, 2, 16, 4, 100, 64, 50,
                                   0, 0, 0, 0) == 4
+    assert lib.awqmi_moe_gemm_f16(fake, fake, fake, fake, fake, fake, fake, fake, 0, 8, 2, 24, 4, 128, 64, 128,
+                                  0, 0, 0, 0) == 7
     assert lib.awqmi_silu_and_mul_f16(fake, fake, 4, 12, 0) == 1
     assert lib.awqmi_moe_sum_f16(fake, fake, 4, 2, 12, 0) == 1
 
@@ -76,6 +78,7 @@ def test_workspace_and_split_k_queries(lib):
             assert need >= 65536 + s * 16 * N * 4
     assert lib.awqmi_gemm_workspace_bytes(512, 8192, 8192, 0) == 65536      # MFMA kernel: no partials
     assert lib.awqmi_gemm_auto_split_k(512, 8192, 8192, 128) == 1
+    assert lib.awqmi_gemm_workspace_bytes(32, 8192, 8192, 8) >= 65536 + 8 * 32 * 8192 * 4
     assert lib.awqmi_moe_align_capacity(8, 128, 16) == (8 + 128 * 15 + 15) // 16 * 16
     assert lib.awqmi_moe_align_capacity(4096, 128, 16) % 16 == 0
 
