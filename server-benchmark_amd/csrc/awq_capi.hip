@@ -249,8 +249,17 @@ int awqmi_moe_topk_softmax_f32(const float* logits, int T, int E, int topk, int 
   if (!logits || !topk_ids || !topk_weights) return AWQMI_NULL_POINTER;
   if (T <= 0 || E <= 0) return AWQMI_BAD_SHAPE;
   if (E > AWQMI_MAX_EXPERTS || topk <= 0 || topk > E || topk > 64) return AWQMI_BAD_ARGUMENT;
-  hipLaunchKernelGGL(moe_topk_softmax_kernel, dim3((T + 3) / 4), dim3(256), 0, (hipStream_t)stream,
-                     logits, T, E, topk, renormalize, topk_ids, topk_weights);
+  const dim3 grid((T + 3) / 4);
+  hipStream_t st = (hipStream_t)stream;
+#define AWQMI_TOPK(P) \
+  hipLaunchKernelGGL(moe_topk_softmax_kernel<P>, grid, dim3(256), 0, st, logits, T, E, topk, renormalize, \
+                     topk_ids, topk_weights)
+  if (E <= 64) AWQMI_TOPK(1);
+  else if (E <= 128) AWQMI_TOPK(2);
+  else if (E <= 256) AWQMI_TOPK(4);
+  else if (E <= 512) AWQMI_TOPK(8);
+  else AWQMI_TOPK(16);
+#undef AWQMI_TOPK
   return launch_status();
 }
 
@@ -267,7 +276,15 @@ int awqmi_moe_align(const int32_t* topk_ids, int n_slots, int E, int tile_m, int
   if (n_slots <= 0 || E <= 0) return AWQMI_BAD_SHAPE;
   if (E > AWQMI_MAX_EXPERTS || tile_m <= 0 || tile_m > 4096) return AWQMI_BAD_ARGUMENT;
   const int cap = (int)awqmi_moe_align_capacity(n_slots, E, tile_m);
-  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(512), (size_t)10 * E * sizeof(int),
+  static std::atomic<bool> align_attr{false};
+  if (!align_attr.load(std::memory_order_acquire)) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(moe_align_kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             (MOE_ALIGN_WAVES + 2) * AWQMI_MAX_EXPERTS * (int)sizeof(int));
+    if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
+    align_attr.store(true, std::memory_order_release);
+  }
+  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)(MOE_ALIGN_WAVES + 2) * E * sizeof(int),
                      (hipStream_t)stream, topk_ids, n_slots, E, tile_m, cap, sorted_token_ids,
                      expert_ids, num_tokens_post_padded);
   return launch_status();

@@ -299,6 +299,9 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
   constexpr int TM = 16 * MB;      // rows per pass
   __shared__ __align__(16) float red[2][16][RS];
   __shared__ int s_last;
+  __shared__ int s_sid[32];     // MoE: slot id of every row of this block (pads: n_slots)
+  __shared__ float s_tw[32];    // MoE: routing weight of the row (1 when not applied)
+  __shared__ int s_rows;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, h = lane >> 4;
   const int cb = blockIdx.x, sp = blockIdx.y;
@@ -313,6 +316,19 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
     qw += (size_t)e * p.w_stride;
     sc += (size_t)e * p.s_stride;
     qz += (size_t)e * p.z_stride;
+    // one global read per row of the block; everything later takes ids / weights from LDS
+    if (tid < 64) {
+      int sid = p.n_slots;
+      if (tid < TM) sid = p.sorted_ids[blk * TM + tid];
+      const bool ok = sid < p.n_slots;
+      if (tid < TM) {
+        s_sid[tid] = sid;
+        s_tw[tid] = (ok && p.topk_w) ? p.topk_w[sid] : 1.f;
+      }
+      const unsigned long long m = __ballot(ok);
+      if (tid == 0) s_rows = __popcll(m);   // valid slots sit at the front of a block
+    }
+    __syncthreads();
   }
 
   // Lanes past the last word column / past the last row read valid memory of column block 0
@@ -328,7 +344,7 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
     if (!MOE) {
       arow = r < p.M ? (size_t)r : 0;
     } else {
-      const int sid = p.sorted_ids[blk * TM + r];
+      const int sid = s_sid[r];
       arow = sid < p.n_slots ? (size_t)(sid / p.a_row_div) : 0;
     }
     w.x_lane[mb] = p.x + arow * p.K + 8 * h;
@@ -352,11 +368,7 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
   const int c_end = (int)((pw + 1) * nchunks / parts);
   w.run(c_begin, c_end);
 
-  int rows_total = p.M;
-  if (MOE) {  // valid slots sit at the front of a block, pads behind them
-    rows_total = 0;
-    for (int m = 0; m < TM; ++m) rows_total += p.sorted_ids[blk * TM + m] < p.n_slots ? 1 : 0;
-  }
+  const int rows_total = MOE ? s_rows : p.M;
   const size_t tile = (size_t)blk * p.ncb + cb;
   const size_t ntiles = (size_t)(MOE ? gridDim.z : 1) * p.ncb;
   constexpr int TILE_F = 16 * NT * 16;   // floats per partial tile (one row block)
@@ -376,11 +388,8 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
       if (!MOE) {
         p.y[(size_t)(mb * 16 + m) * p.N + col] = (half_t)v;
       } else {
-        const int sid = p.sorted_ids[blk * TM + mb * 16 + m];
-        if (sid < p.n_slots) {
-          if (p.topk_w) v *= p.topk_w[sid];
-          p.y[(size_t)sid * p.N + col] = (half_t)v;
-        }
+        const int sid = s_sid[mb * 16 + m];
+        if (sid < p.n_slots) p.y[(size_t)sid * p.N + col] = (half_t)(v * s_tw[mb * 16 + m]);
       }
     }
   };

@@ -8,7 +8,8 @@
 namespace awqmi {
 
 // One wave per token.  Selection runs on the raw logits (softmax is monotonic), ties go to
-// the lowest expert id.  E <= 1024.
+// the lowest expert id.  PER = experts per lane (E <= 64 * PER).
+template <int PER>
 __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __restrict__ logits, int T,
                                                                int E, int topk, int renorm,
                                                                int* __restrict__ ids,
@@ -16,7 +17,6 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __re
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
-  constexpr int PER = 16;  // 64 * 16 = 1024 experts at most
   float v[PER];
   float mx = -INFINITY;
 #pragma unroll
@@ -66,25 +66,30 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __re
   }
 }
 
-// Single workgroup of 8 waves.  Dynamic LDS: cnt[8][E] + padded[E] + start[E].
+// Single workgroup of 16 waves.  Dynamic LDS: cnt[16][E] + padded[E] + start[E].
 // Wave w owns the contiguous slice [w*seg, (w+1)*seg) of the flat slot list, so placing
-// slices in wave order and slots in index order inside a slice gives a stable sort.
-__global__ __launch_bounds__(512) void moe_align_kernel(const int* __restrict__ ids, int n, int E,
-                                                        int tile_m, int cap,
-                                                        int* __restrict__ sorted,
-                                                        int* __restrict__ expert_ids,
-                                                        int* __restrict__ npp) {
+// slices in wave order and slots in index order inside a slice gives a stable sort.  Inside a
+// batch of 64 slots a lane's rank among equal expert ids is a count over lower lanes (64
+// scalar broadcasts, no LDS round trips); the running position per (wave, expert) lives in
+// LDS and is bumped by one LDS atomic per slot after all lanes of the batch have read it.
+constexpr int MOE_ALIGN_WAVES = 16;
+__global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int n, int E,
+                                                         int tile_m, int cap,
+                                                         int* __restrict__ sorted,
+                                                         int* __restrict__ expert_ids,
+                                                         int* __restrict__ npp) {
   extern __shared__ int sm[];
-  int* cnt = sm;             // [8][E], later the running write position
-  int* padded = sm + 8 * E;  // [E]
-  int* start = padded + E;   // [E]
+  constexpr int NWV = MOE_ALIGN_WAVES;
+  int* cnt = sm;               // [NWV][E], later the running write position
+  int* padded = sm + NWV * E;  // [E]
+  int* start = padded + E;     // [E]
   __shared__ int s_total;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 
-  for (int i = tid; i < 8 * E; i += 512) cnt[i] = 0;
+  for (int i = tid; i < NWV * E; i += 1024) cnt[i] = 0;
   __syncthreads();
 
-  const int seg = ((n + 8 * 64 - 1) / (8 * 64)) * 64;
+  const int seg = ((n + NWV * 64 - 1) / (NWV * 64)) * 64;
   const int sb = wave * seg, se = min(n, sb + seg);
   for (int i = sb + lane; i < se; i += 64) {
     const int e = ids[i];
@@ -92,46 +97,61 @@ __global__ __launch_bounds__(512) void moe_align_kernel(const int* __restrict__ 
   }
   __syncthreads();
 
-  for (int e = tid; e < E; e += 512) {
+  for (int e = tid; e < E; e += 1024) {
     int tot = 0;
-    for (int w = 0; w < 8; ++w) tot += cnt[w * E + e];
+    for (int w = 0; w < NWV; ++w) tot += cnt[w * E + e];
     padded[e] = (tot + tile_m - 1) / tile_m * tile_m;
   }
   __syncthreads();
-  if (tid == 0) {
-    int pos = 0;
-    for (int e = 0; e < E; ++e) { start[e] = pos; pos += padded[e]; }
-    s_total = pos;
-    npp[0] = pos;
+  if (wave == 0) {   // exclusive prefix sum of padded[] by one wave: lane owns a contiguous run
+    const int per = (E + 63) / 64;
+    int local = 0;
+    for (int k = 0; k < per; ++k) {
+      const int e = lane * per + k;
+      if (e < E) local += padded[e];
+    }
+    int incl = local;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int v = __shfl_up(incl, o);
+      if (lane >= o) incl += v;
+    }
+    int pos = incl - local;
+    for (int k = 0; k < per; ++k) {
+      const int e = lane * per + k;
+      if (e < E) { start[e] = pos; pos += padded[e]; }
+    }
+    if (lane == 63) { s_total = incl; npp[0] = incl; }
   }
   __syncthreads();
   const int total = s_total;
-  for (int e = tid; e < E; e += 512) {
+  for (int e = tid; e < E; e += 1024) {
     int pos = start[e];
     const int s0 = pos;
-    for (int w = 0; w < 8; ++w) { const int c = cnt[w * E + e]; cnt[w * E + e] = pos; pos += c; }
+    for (int w = 0; w < NWV; ++w) { const int c = cnt[w * E + e]; cnt[w * E + e] = pos; pos += c; }
     for (int i = pos; i < s0 + padded[e]; ++i) sorted[i] = n;            // pad entries
     for (int b = 0; b < padded[e] / tile_m; ++b) expert_ids[s0 / tile_m + b] = e;
   }
-  for (int i = total + tid; i < cap; i += 512) sorted[i] = n;           // unused tail
-  for (int i = total / tile_m + tid; i < cap / tile_m; i += 512) expert_ids[i] = -1;
+  for (int i = total + tid; i < cap; i += 1024) sorted[i] = n;           // unused tail
+  for (int i = total / tile_m + tid; i < cap / tile_m; i += 1024) expert_ids[i] = -1;
   __syncthreads();
 
   for (int i0 = sb; i0 < se; i0 += 64) {
     const int i = i0 + lane;
     int e = i < se ? ids[i] : -1;
     const bool valid = e >= 0 && e < E;
-    unsigned long long remaining = __ballot(valid);
-    while (remaining) {
-      const int leader = __ffsll((long long)remaining) - 1;
-      const int e0 = __shfl(e, leader);
-      const bool mine = valid && e == e0;
-      const unsigned long long mask = __ballot(mine);
-      const int rank = __popcll(mask & ((1ull << lane) - 1ull));
-      const int base = cnt[wave * E + e0];
-      if (mine) sorted[base + rank] = i;
-      if (lane == leader) cnt[wave * E + e0] = base + __popcll(mask);
-      remaining &= ~mask;
+    if (!valid) e = -1 - lane;     // never equal to another lane's id
+    int rank = 0;
+    for (int l = 0; l < 63; ++l) {
+      const int el = __builtin_amdgcn_readlane(e, l);
+      rank += (el == e && l < lane) ? 1 : 0;
+    }
+    int base = 0;
+    if (valid) base = cnt[wave * E + e];
+    __builtin_amdgcn_wave_barrier();
+    if (valid) {
+      sorted[base + rank] = i;
+      atomicAdd(&cnt[wave * E + e], 1);
     }
   }
 }

@@ -214,7 +214,7 @@ def moe_sum(x: torch.Tensor, T: int, topk: int) -> torch.Tensor:
 
 
 def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Tensor, topk: int,
-                  renormalize: bool = True) -> torch.Tensor:
+                  renormalize: bool = True, block_size: int | None = None) -> torch.Tensor:
     """One AWQ MoE block: route -> align -> grouped GEMM (w13) -> SiLU*up -> grouped GEMM (w2,
     scaled by the routing weight) -> sum over slots.  w13 / w2 are (qweight, scales, qzeros)
     with a leading expert dimension; w13 columns are [gate | up]."""
@@ -222,9 +222,9 @@ def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Ten
     E = w13[0].shape[0]
     topk_w, topk_ids = topk_softmax(gating_output.float().contiguous(), topk, renormalize)
     n = T * topk
-    # 32-row blocks once an expert sees more than ~16 slots on average: one pass over its
-    # weights instead of two
-    bs = 32 if n > 16 * E else MOE_TILE_M
+    # 16-row blocks measured faster than 32-row blocks at every token count tried (the
+    # two-row-block instantiation of the skinny kernel is issue-bound)
+    bs = block_size if block_size is not None else MOE_TILE_M
     sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, bs, E)
     h13 = moe_awq_gemm(hidden_states, *w13, sorted_ids, expert_ids, npp, n, topk, block_size=bs)
     act = silu_and_mul(h13)
