@@ -102,7 +102,8 @@ def main():
         W[name] = [make_weights(K, N, G, dev, gen) for _ in range(NCOPY)]
         X[name] = {M: torch.randn((M, K), device=dev, generator=gen).to(torch.float16) for M in Ms}
         Y[name] = {M: torch.empty((M, N), dtype=torch.float16, device=dev) for M in Ms}
-    ws_bytes = max(lib.awqmi_gemm_workspace_bytes(M, K, N, args.split_k) for _, K, N in layers for M in Ms)
+    ws_bytes = max(lib.awqmi_gemm_workspace_bytes(M, K, N, args.split_k) for _, K, N in layers
+                   for M in tuple(Ms) + tuple(workloads.PREFILL_M))
     ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
     torch.cuda.synchronize()
     log(f"[bench] inputs resident after {time.time() - t0:.1f}s, "

@@ -179,6 +179,16 @@ def test_gemm_prefill(sba, gpu, M, K, N, G):
     _check_gemm(sba, gpu, x, qw, s, qz, K if G <= 0 else G, 0, tag="prefill")
 
 
+@pytest.mark.parametrize("M,K,N", [(512, 1024, 1280), (300, 2048, 520), (2048, 512, 5120), (768, 1536, 8192 + 256)])
+def test_gemm_prefill_partial_rounds(sba, gpu, M, K, N):
+    """Tile counts that are not a multiple of the CU count, ragged last row / column tiles;
+    two runs must agree bit for bit."""
+    x, qw, s, qz = _np_case(M, K, N, 128, seed=M + N)
+    y1 = _check_gemm(sba, gpu, x, qw, s, qz, 128, 0, tag="prefill-rounds")
+    y2 = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), 0).cpu().numpy()
+    assert np.array_equal(y1.view(np.uint16), y2.view(np.uint16))      # deterministic
+
+
 @pytest.mark.parametrize("M,K,N,G", [(3, 96, 40, 32), (20, 100, 16, 50), (2, 24, 8, 8)])
 def test_gemm_generic_fallback(sba, gpu, M, K, N, G):
     x, qw, s, qz = _np_case(M, K, N, G, seed=5)
