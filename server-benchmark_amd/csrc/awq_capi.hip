@@ -92,29 +92,6 @@ void launch_gemv(const GemvParams& p, dim3 grid, hipStream_t st) {
 // rows the skinny kernel takes in one awq_gemm call (passes of up to 32 rows)
 constexpr int SKINNY_MAX_M = 64;
 
-// Work split of the MFMA kernel: whole rounds of 256 tiles run data-parallel; a last round
-// that would leave more than a fifth of the CUs idle (and any launch of fewer than 256
-// tiles) is split stream-K over up to 256 workgroups, at most 8 contributors per tile and
-// at least 4 k-tiles per workgroup.
-struct MfmaPlan { int dp_tiles, sk_tiles, sk_wgs; size_t part_bytes; };
-MfmaPlan plan_mfma(int M, int K, int N) {
-  const int mt = (M + PF_BM - 1) / PF_BM, nt = (N + PF_BN - 1) / PF_BN;
-  const int tiles = mt * nt, KT = K / PF_BK;
-  MfmaPlan pl{tiles, 0, 0, 0};
-  const int rem = tiles % 256;
-  if (rem == 0 || rem >= 208) return pl;
-  long long wgs = (long long)rem * KT / 4;
-  if (wgs > 256) wgs = 256;
-  if (wgs > 8LL * rem) wgs = 8LL * rem;
-  wgs = wgs / 8 * 8;
-  if (wgs < 8 || wgs <= rem) return pl;      // nothing to gain
-  pl.dp_tiles = tiles - rem;
-  pl.sk_tiles = rem;
-  pl.sk_wgs = (int)wgs;
-  pl.part_bytes = (size_t)pl.sk_wgs * 2 * PF_SK_SLOT_FLOATS * sizeof(float);
-  return pl;
-}
-
 }  // namespace
 
 extern "C" {
@@ -174,10 +151,7 @@ int awqmi_gemm_auto_split_k(int M, int K, int N, int group) {
 
 size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
   if (M <= 0 || K <= 0 || N <= 0) return 0;
-  if (M > SKINNY_MAX_M) {
-    if (K % PF_BK != 0) return AWQMI_WS_COUNTER_BYTES;
-    return AWQMI_WS_COUNTER_BYTES + plan_mfma(M, K, N).part_bytes;
-  }
+  if (M > SKINNY_MAX_M) return AWQMI_WS_COUNTER_BYTES;
   int s = split_k;
   if (s <= 0) s = (K % 128 == 0) ? pick_split_k(M, K, N, 128, 1) : 1;
   return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, s, 1, 32);
@@ -257,23 +231,11 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     p.gshift = 0;
     if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
     p.mt = (M + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
-    p.total = p.mt * p.nt;
-    MfmaPlan pl = plan_mfma(M, K, N);
-    // stream-K needs the caller's workspace (counters + partial tiles); without it every
-    // tile runs data-parallel
-    if (pl.sk_wgs > 0 && (!workspace || !aligned16(workspace) ||
-                          workspace_bytes < AWQMI_WS_COUNTER_BYTES + pl.part_bytes))
-      pl = MfmaPlan{p.total, 0, 0, 0};
-    p.dp_tiles = pl.dp_tiles; p.sk_tiles = pl.sk_tiles; p.sk_wgs = pl.sk_wgs;
-    p.dp_per_xcd = (pl.dp_tiles + 7) / 8; p.dp_grid = p.dp_per_xcd * 8;
-    p.sk_cnt = reinterpret_cast<int*>(workspace);
-    p.sk_part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
-                          : nullptr;
-    const dim3 grid(p.dp_grid + p.sk_wgs);
+    p.total = p.mt * p.nt; p.per_xcd = (p.total + 7) / 8;
     if (pow2g)
-      hipLaunchKernelGGL(awq_gemm_mfma_kernel<true>, grid, dim3(256), PF_LDS_BYTES, st, p);
+      hipLaunchKernelGGL(awq_gemm_mfma_kernel<true>, dim3(p.per_xcd * 8), dim3(256), PF_LDS_BYTES, st, p);
     else
-      hipLaunchKernelGGL(awq_gemm_mfma_kernel<false>, grid, dim3(256), PF_LDS_BYTES, st, p);
+      hipLaunchKernelGGL(awq_gemm_mfma_kernel<false>, dim3(p.per_xcd * 8), dim3(256), PF_LDS_BYTES, st, p);
     return launch_status();
   }
 

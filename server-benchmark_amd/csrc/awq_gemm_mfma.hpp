@@ -36,19 +36,8 @@ struct MfmaGemmParams {
   int gshift;     // log2(G) when G is a power of two (kernel instantiation POW2G)
   int mt, nt;     // tile counts
   int total;      // mt * nt
-  // Work split.  Tiles [0, dp_tiles) are data-parallel: one workgroup per tile, launch ids
-  // [0, dp_grid).  The remaining sk_tiles tiles are split stream-K style: their
-  // sk_tiles * (K / 64) k-tile iterations are dealt out evenly over sk_wgs workgroups
-  // (launch ids from dp_grid on), so the last, partly filled round of tiles costs its share
-  // of a round instead of a whole one.  A tile with several contributors is finished by
-  // whichever contributor arrives last, from fp32 partials in the workspace.
-  int dp_tiles, dp_grid, dp_per_xcd;
-  int sk_tiles, sk_wgs;
-  float* sk_part;   // [sk_wgs][2][256 * 256] fp32
-  int* sk_cnt;      // [sk_tiles] arrival counters (zero before and after the launch)
+  int per_xcd;    // ceil(total / 8)
 };
-
-constexpr int PF_SK_SLOT_FLOATS = 256 * 256;
 
 constexpr int PF_BM = 256, PF_BN = 256, PF_BK = 64;
 constexpr int PF_ROW_BYTES = PF_BK * 2;                       // 128 B = eight 16-byte slots
@@ -61,17 +50,6 @@ constexpr int PF_LDS_BYTES = 4 * PF_TILE_BYTES;               // A0 A1 B0 B1
 // word columns a wave's neighbouring lanes dequantise (rows 8 apart) do too (conflict-free
 // stores of the dequantised W tile).
 __device__ __forceinline__ int pf_swz(int row) { return (row ^ (row >> 3)) & 7; }
-
-// 8-byte device-coherent store / load of two floats (relaxed, agent scope)
-__device__ __forceinline__ void st_coherent2(float* p, float a, float b) {
-  const float2 v = {a, b};
-  __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), __builtin_bit_cast(unsigned long long, v),
-                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float2 ld_coherent2(const float* p) {
-  return __builtin_bit_cast(float2, __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p),
-                                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-}
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* base, size_t bytes) {
   const uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)bytes;
@@ -88,46 +66,20 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int id = blockIdx.x;
-  const int KT = p.K / PF_BK;
+  const int nid = (id & 7) * p.per_xcd + (id >> 3);
+  if (nid >= p.total) return;
+  const int gsize = 8 * p.nt;
+  const int first_m = (nid / gsize) * 8;
+  const int gm = min(p.mt - first_m, 8);
+  const int mt_i = first_m + (nid % gsize) % gm;
+  const int nt_i = (nid % gsize) / gm;
+  const int m0 = mt_i * PF_BM, n0 = nt_i * PF_BN;
   const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
-  __shared__ int s_last;
-
-  // this workgroup's range of (tile, k-tile) iterations, tile-major
-  long long it0, it1;
-  int sk_id = -1;
-  if (id < p.dp_grid) {
-    const int nid = (id & 7) * p.dp_per_xcd + (id >> 3);
-    if (nid >= p.dp_tiles) return;
-    it0 = (long long)nid * KT;
-    it1 = it0 + KT;
-  } else {
-    const int j = id - p.dp_grid;
-    sk_id = (j & 7) * (p.sk_wgs >> 3) + (j >> 3);     // contiguous ranges per XCD
-    const long long I = (long long)p.sk_tiles * KT;
-    it0 = (long long)p.dp_tiles * KT + I * sk_id / p.sk_wgs;
-    it1 = (long long)p.dp_tiles * KT + I * (sk_id + 1) / p.sk_wgs;
-  }
 
   const __amdgpu_buffer_rsrc_t rx = pf_rsrc(p.x, (size_t)p.M * p.K * 2);
   const __amdgpu_buffer_rsrc_t rw = pf_rsrc(p.qw, (size_t)p.K * p.NW * 4);
   const __amdgpu_buffer_rsrc_t rz = pf_rsrc(p.qz, (size_t)(p.K / p.G) * p.NW * 4);
   const __amdgpu_buffer_rsrc_t rs = pf_rsrc(p.sc, (size_t)(p.K / p.G) * p.N * 2);
-
-  bool first_seg = true;
-  for (long long it = it0; it < it1;) {
-  const int tile_lin = (int)(it / KT);
-  const int kb = (int)(it % KT);
-  const int ke = (int)min((long long)KT, kb + (it1 - it));
-  it += ke - kb;
-  // tile order: groups of eight row tiles, column tiles inside a group
-  const int gsize = 8 * p.nt;
-  const int first_m = (tile_lin / gsize) * 8;
-  const int gm = min(p.mt - first_m, 8);
-  const int mt_i = first_m + (tile_lin % gsize) % gm;
-  const int nt_i = (tile_lin % gsize) / gm;
-  const int m0 = mt_i * PF_BM, n0 = nt_i * PF_BN;
-  if (!first_seg) __syncthreads();   // the previous segment's last fragment reads are done
-  first_seg = false;
 
   // ---- global -> LDS roles -------------------------------------------------------------
   // X tile: thread (a_row + 32 i, a_seg) moves 16 bytes; rows past M re-read row M - 1 (their
@@ -174,6 +126,8 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   uint32_t wreg[2][8];  // two W tiles in flight (parity of the k-tile)
   uint32_t zreg[2];
   u4v sreg[2];
+  const int KT = p.K / PF_BK;
+
   auto gload_a = [&](int kt) {
     const int so = kt * (PF_BK * 2);
 #pragma unroll
@@ -271,7 +225,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   // end re-read the last tile and are never used.
   auto body = [&](int kt, auto PTAG) {
     constexpr int PAR = decltype(PTAG)::value;
-    const int kt2 = min(kt + 2, ke - 1);
+    const int kt2 = min(kt + 2, KT - 1);
 
     // phase 1: X(kt+1) -> LDS, W(kt+2) -> registers, byte 0 of W(kt+1)
     mfma_step(0);
@@ -309,80 +263,24 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   };
 
   // prologue: tile 0 into LDS buffer 0, tile 1 into registers
-  gload_a(kb);
-  gload_w(kb, 0);
+  gload_a(0);
+  gload_w(0, 0);
   store_a(0);
   dq_byte(0, 0, I0{});
   dq_byte(0, 0, I1{});
   dq_byte(0, 0, I2{});
   dq_byte(0, 0, I3{});
-  gload_a(min(kb + 1, ke - 1));
-  gload_w(min(kb + 1, ke - 1), 1);
+  gload_a(min(1, KT - 1));
+  gload_w(min(1, KT - 1), 1);
   __syncthreads();
   load_frags(0, 0, 0);
   __builtin_amdgcn_sched_barrier(0);
-  int kt = kb;
-  for (; kt + 1 < ke; kt += 2) {
+  int kt = 0;
+  for (; kt + 1 < KT; kt += 2) {
     body(kt, I0{});
     body(kt + 1, I1{});
   }
-  if (kt < ke) body(kt, I0{});
-
-  // ---- stream-K fix-up: a segment that does not span all of K is a partial sum ----------
-  if (ke - kb < KT) {
-    const int tl = tile_lin - p.dp_tiles;
-    const long long I = (long long)p.sk_tiles * KT;
-    const long long W = p.sk_wgs;
-    // contributors of this tile: owners of its first and last iteration
-    const long long ta = (long long)tl * KT, tb = ta + KT - 1;
-    const int s_first = (int)(((ta + 1) * W - 1) / I);
-    const int s_last_c = (int)(((tb + 1) * W - 1) / I);
-    const int ncontrib = s_last_c - s_first + 1;
-    // slot 0: the segment at the start of a workgroup's range, slot 1: the one at its end
-    auto slot_of = [&](int sid) -> const float* {
-      const long long r0 = I * sid / W;
-      const int which = (r0 >= ta && r0 <= tb) ? 0 : 1;
-      return p.sk_part + ((size_t)sid * 2 + which) * PF_SK_SLOT_FLOATS;
-    };
-    float* mine = const_cast<float*>(slot_of(sk_id));
-    // layout [pair of accumulator registers][thread]: coalesced 8-byte accesses
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const int q = ((i * 4 + j) * 16 + r) >> 1;
-          st_coherent2(mine + ((size_t)q * 256 + tid) * 2, acc[i][j][r], acc[i][j][r + 1]);
-        }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (tid == 0) s_last = (atomicAdd(p.sk_cnt + tl, 1) == ncontrib - 1);
-    __syncthreads();
-    if (!s_last) continue;            // somebody else finishes this tile
-    // Sum every contributor's partial (own included, from memory) in contributor order, so
-    // the result does not depend on who arrived last; fp16 result straight to y.
-    // Pair q of thread tid: tile (i, j) = q / 8, registers r = 2 (q % 8), r + 1.
-    const int col_l = lane & 31, row_l = 4 * (lane >> 5);
-#pragma unroll 2
-    for (int q = 0; q < 128; ++q) {
-      float v0 = 0.f, v1 = 0.f;
-      for (int sid = s_first; sid <= s_last_c; ++sid) {
-        const float2 t = ld_coherent2(slot_of(sid) + ((size_t)q * 256 + tid) * 2);
-        v0 += t.x;
-        v1 += t.y;
-      }
-      const int ij = q >> 3, r = (q & 7) * 2;
-      const int col = n0 + wn + 32 * (ij & 3) + col_l;
-      const int row = m0 + wm + 32 * (ij >> 2) + 8 * (r >> 2) + row_l + (r & 3);
-      if (col < p.N) {
-        if (row < p.M) p.y[(size_t)row * p.N + col] = (half_t)v0;
-        if (row + 1 < p.M) p.y[(size_t)(row + 1) * p.N + col] = (half_t)v1;
-      }
-    }
-    if (tid == 0) __hip_atomic_store(p.sk_cnt + tl, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    continue;
-  }
+  if (kt < KT) body(kt, I0{});
 
   // D[i][j] of a 32x32 tile: j = lane % 32, i = 8 * (r / 4) + 4 * (lane / 32) + r % 4
   const int col_l = lane & 31, row_l = 4 * (lane >> 5);
@@ -398,7 +296,6 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
         if (row < p.M) p.y[(size_t)row * p.N + col] = (half_t)acc[i][j][r];
       }
     }
-  }   // segments
 }
 
 }  // namespace awqmi
