@@ -92,6 +92,27 @@ void launch_gemv(const GemvParams& p, dim3 grid, hipStream_t st) {
 // rows the skinny kernel takes in one awq_gemm call (passes of up to 32 rows)
 constexpr int SKINNY_MAX_M = 64;
 
+// Work split of the MFMA kernel: whole rounds of 256 tiles run one workgroup per tile; a
+// last round of fewer than 129 tiles (and any launch that small) is split in K over
+// floor(256 / tiles) workgroups per tile (at most 8, at least 8 k-tiles each).
+struct MfmaPlan { int dp_tiles, sk_tiles, sk_split; size_t part_bytes; };
+MfmaPlan plan_mfma(int M, int K, int N) {
+  const int mt = (M + PF_BM - 1) / PF_BM, nt = (N + PF_BN - 1) / PF_BN;
+  const int tiles = mt * nt, KT = K / PF_BK;
+  MfmaPlan pl{tiles, 0, 1, 0};
+  const int rem = tiles % 256;
+  if (rem == 0) return pl;
+  int c = 256 / rem;
+  if (c > 8) c = 8;
+  while (c > 1 && KT / c < 8) --c;
+  if (c < 2) return pl;
+  pl.dp_tiles = tiles - rem;
+  pl.sk_tiles = rem;
+  pl.sk_split = c;
+  pl.part_bytes = (size_t)rem * c * PF_SK_SLOT_FLOATS * sizeof(float);
+  return pl;
+}
+
 }  // namespace
 
 extern "C" {
@@ -151,7 +172,10 @@ int awqmi_gemm_auto_split_k(int M, int K, int N, int group) {
 
 size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
   if (M <= 0 || K <= 0 || N <= 0) return 0;
-  if (M > SKINNY_MAX_M) return AWQMI_WS_COUNTER_BYTES;
+  if (M > SKINNY_MAX_M) {
+    if (K % PF_BK != 0) return AWQMI_WS_COUNTER_BYTES;
+    return AWQMI_WS_COUNTER_BYTES + plan_mfma(M, K, N).part_bytes;
+  }
   int s = split_k;
   if (s <= 0) s = (K % 128 == 0) ? pick_split_k(M, K, N, 128, 1) : 1;
   return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, s, 1, 32);
@@ -231,11 +255,23 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     p.gshift = 0;
     if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
     p.mt = (M + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
-    p.total = p.mt * p.nt; p.per_xcd = (p.total + 7) / 8;
+    p.total = p.mt * p.nt;
+    MfmaPlan pl = plan_mfma(M, K, N);
+    // the K split needs the caller's workspace (counters + partial tiles); without it every
+    // tile runs on one workgroup
+    if (pl.sk_tiles > 0 && (!workspace || !aligned16(workspace) ||
+                            workspace_bytes < AWQMI_WS_COUNTER_BYTES + pl.part_bytes))
+      pl = MfmaPlan{p.total, 0, 1, 0};
+    p.dp_tiles = pl.dp_tiles; p.sk_tiles = pl.sk_tiles; p.sk_split = pl.sk_split;
+    p.per_xcd = (pl.dp_tiles + 7) / 8;
+    p.sk_cnt = reinterpret_cast<int*>(workspace);
+    p.sk_part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
+                          : nullptr;
+    const dim3 grid(p.per_xcd * 8 + p.sk_tiles * p.sk_split);
     if (pow2g)
-      hipLaunchKernelGGL(awq_gemm_mfma_kernel<true>, dim3(p.per_xcd * 8), dim3(256), PF_LDS_BYTES, st, p);
+      hipLaunchKernelGGL(awq_gemm_mfma_kernel<true>, grid, dim3(256), PF_LDS_BYTES, st, p);
     else
-      hipLaunchKernelGGL(awq_gemm_mfma_kernel<false>, dim3(p.per_xcd * 8), dim3(256), PF_LDS_BYTES, st, p);
+      hipLaunchKernelGGL(awq_gemm_mfma_kernel<false>, grid, dim3(256), PF_LDS_BYTES, st, p);
     return launch_status();
   }
 

@@ -36,8 +36,18 @@ struct MfmaGemmParams {
   int gshift;     // log2(G) when G is a power of two (kernel instantiation POW2G)
   int mt, nt;     // tile counts
   int total;      // mt * nt
-  int per_xcd;    // ceil(total / 8)
+  int per_xcd;    // ceil(dp_tiles / 8)
+  // Work split.  Tiles [0, dp_tiles) run one workgroup per tile over all of K (launch ids
+  // [0, 8 * per_xcd)).  The remaining sk_tiles tiles (a last round that would leave most CUs
+  // idle) are split in K over sk_split workgroups each (launch ids from 8 * per_xcd on,
+  // tile-major); the contributor that arrives last sums the fp32 partial tiles in the
+  // workspace in fixed order and writes the result.
+  int dp_tiles, sk_tiles, sk_split;
+  float* sk_part;   // [sk_tiles][sk_split][256 * 256] fp32
+  int* sk_cnt;      // [sk_tiles] arrival counters (zero before and after the launch)
 };
+
+constexpr int PF_SK_SLOT_FLOATS = 256 * 256;
 
 constexpr int PF_BM = 256, PF_BN = 256, PF_BK = 64;
 constexpr int PF_ROW_BYTES = PF_BK * 2;                       // 128 B = eight 16-byte slots
@@ -66,8 +76,19 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int id = blockIdx.x;
-  const int nid = (id & 7) * p.per_xcd + (id >> 3);
-  if (nid >= p.total) return;
+  const int KT = p.K / PF_BK;
+  __shared__ int s_last;
+  int nid, kb = 0, ke = KT, part = -1;
+  if (id < 8 * p.per_xcd) {
+    nid = (id & 7) * p.per_xcd + (id >> 3);
+    if (nid >= p.dp_tiles) return;
+  } else {
+    const int j = id - 8 * p.per_xcd;
+    nid = p.dp_tiles + j / p.sk_split;
+    part = j % p.sk_split;
+    kb = (int)((long long)KT * part / p.sk_split);
+    ke = (int)((long long)KT * (part + 1) / p.sk_split);
+  }
   const int gsize = 8 * p.nt;
   const int first_m = (nid / gsize) * 8;
   const int gm = min(p.mt - first_m, 8);
@@ -126,8 +147,6 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   uint32_t wreg[2][8];  // two W tiles in flight (parity of the k-tile)
   uint32_t zreg[2];
   u4v sreg[2];
-  const int KT = p.K / PF_BK;
-
   auto gload_a = [&](int kt) {
     const int so = kt * (PF_BK * 2);
 #pragma unroll
@@ -225,7 +244,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   // end re-read the last tile and are never used.
   auto body = [&](int kt, auto PTAG) {
     constexpr int PAR = decltype(PTAG)::value;
-    const int kt2 = min(kt + 2, KT - 1);
+    const int kt2 = min(kt + 2, ke - 1);
 
     // phase 1: X(kt+1) -> LDS, W(kt+2) -> registers, byte 0 of W(kt+1)
     mfma_step(0);
@@ -263,24 +282,83 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   };
 
   // prologue: tile 0 into LDS buffer 0, tile 1 into registers
-  gload_a(0);
-  gload_w(0, 0);
+  gload_a(kb);
+  gload_w(kb, 0);
   store_a(0);
   dq_byte(0, 0, I0{});
   dq_byte(0, 0, I1{});
   dq_byte(0, 0, I2{});
   dq_byte(0, 0, I3{});
-  gload_a(min(1, KT - 1));
-  gload_w(min(1, KT - 1), 1);
+  gload_a(min(kb + 1, ke - 1));
+  gload_w(min(kb + 1, ke - 1), 1);
   __syncthreads();
   load_frags(0, 0, 0);
   __builtin_amdgcn_sched_barrier(0);
-  int kt = 0;
-  for (; kt + 1 < KT; kt += 2) {
+  int kt = kb;
+  for (; kt + 1 < ke; kt += 2) {
     body(kt, I0{});
     body(kt + 1, I1{});
   }
-  if (kt < KT) body(kt, I0{});
+  if (kt < ke) body(kt, I0{});
+
+  // ---- split-K tiles: fp32 partial to the workspace, last arriver finishes the tile ------
+  if (part >= 0) {
+    const int tl = nid - p.dp_tiles;
+    float* tile_base = p.sk_part + (size_t)tl * p.sk_split * PF_SK_SLOT_FLOATS;
+    float* mine = tile_base + (size_t)part * PF_SK_SLOT_FLOATS;
+    // layout [group of four accumulator registers][thread]: coalesced 16-byte accesses
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; r += 4) {
+          const int q = ((i * 4 + j) * 16 + r) >> 2;
+          const f4 v = {acc[i][j][r], acc[i][j][r + 1], acc[i][j][r + 2], acc[i][j][r + 3]};
+          *reinterpret_cast<f4*>(mine + ((size_t)q * 256 + tid) * 4) = v;
+        }
+    // These workgroups live for hundreds of microseconds, so one release / acquire fence
+    // pair per workgroup (an L2 write-back, then an invalidate in the finisher) is cheap
+    // here, and the partial tiles can use ordinary cached 16-byte accesses.
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) s_last = (atomicAdd(p.sk_cnt + tl, 1) == p.sk_split - 1);
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    // sum in part order, own part included from memory: the result does not depend on who
+    // arrived last.  Group q of thread tid: tile (i, j) = q / 4, registers 4 (q % 4) ...
+    const int col_l = lane & 31, row_l = 4 * (lane >> 5);
+    const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
+    for (int q0 = 0; q0 < 64; q0 += 8) {   // eight groups x sk_split loads in flight
+      f4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = f4{0.f, 0.f, 0.f, 0.f};
+      for (int s = 0; s < p.sk_split; ++s) {
+        f4 t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          t[u] = *reinterpret_cast<const f4*>(tile_base + (size_t)s * PF_SK_SLOT_FLOATS +
+                                              ((size_t)(q0 + u) * 256 + tid) * 4);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] += t[u];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int q = q0 + u;
+        const int ij = q >> 2, r = (q & 3) * 4;
+        const int col = n0 + wn + 32 * (ij & 3) + col_l;
+        const int row = m0 + wm + 32 * (ij >> 2) + 8 * (r >> 2) + row_l;
+        if (col < p.N) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (row + e < p.M) p.y[(size_t)(row + e) * p.N + col] = (half_t)v[u][e];
+        }
+      }
+    }
+    if (tid == 0) p.sk_cnt[tl] = 0;
+    return;
+  }
 
   // D[i][j] of a 32x32 tile: j = lane % 32, i = 8 * (r / 4) + 4 * (lane / 32) + r % 4
   const int col_l = lane & 31, row_l = 4 * (lane >> 5);

@@ -76,7 +76,8 @@ def test_workspace_and_split_k_queries(lib):
         assert need >= 65536
         if s > 1:
             assert need >= 65536 + s * 16 * N * 4
-    assert lib.awqmi_gemm_workspace_bytes(512, 8192, 8192, 0) == 65536      # MFMA kernel: no partials
+    assert lib.awqmi_gemm_workspace_bytes(8192, 8192, 8192, 0) == 65536     # whole rounds: no partials
+    assert lib.awqmi_gemm_workspace_bytes(512, 8192, 8192, 0) == 65536 + 64 * 4 * 256 * 256 * 4   # K split
     assert lib.awqmi_gemm_auto_split_k(512, 8192, 8192, 128) == 1
     assert lib.awqmi_gemm_workspace_bytes(32, 8192, 8192, 8) >= 65536 + 8 * 32 * 8192 * 4
     assert lib.awqmi_moe_align_capacity(8, 128, 16) == (8 + 128 * 15 + 15) // 16 * 16
