@@ -367,6 +367,9 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
   const int c_begin = (int)(pw * nchunks / parts);
   const int c_end = (int)((pw + 1) * nchunks / parts);
   w.run(c_begin, c_end);
+#if defined(AWQMI_LAB_EPI) && AWQMI_LAB_EPI == 4
+  if (p.M != 12345) return;
+#endif
 
   const int rows_total = MOE ? s_rows : p.M;
   const size_t tile = (size_t)blk * p.ncb + cb;
@@ -374,23 +377,35 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
   constexpr int TILE_F = 16 * NT * 16;   // floats per partial tile (one row block)
   const bool split = p.split_k > 1;
 
-  // tile-major LDS (red[0], optionally + red[1]) -> row-major fp16 output of row block mb
+  // tile-major LDS (red[0], optionally + red[1]) -> row-major fp16 output of row block mb;
+  // one thread gathers the eight columns of a packed word and stores them as 16 bytes
   auto emit = [&](int mb, int rows, bool two) {
-    for (int i = tid; i < rows * CB; i += 256) {
-      const int m = i / CB, cl = i % CB;
-      const int wl = cl >> 3;                 // word within the block
+    constexpr int WPB = 16 * WPL;   // packed words per row of the block
+    for (int it = tid; it < rows * WPB; it += 256) {
+      const int m = it / WPB, wl = it % WPB;
       const int jj = wl / WPL, ww = wl % WPL;
-      const int t = ww * 8 + awq_nibble_of_col(cl & 7);
-      const int col = cb * CB + cl;
-      float v = red[0][m][t * 16 + jj];
-      if (two) v += red[1][m][t * 16 + jj];
+      const int col = cb * CB + wl * 8;
       if (col >= p.N) continue;
-      if (!MOE) {
-        p.y[(size_t)(mb * 16 + m) * p.N + col] = (half_t)v;
-      } else {
-        const int sid = s_sid[mb * 16 + m];
-        if (sid < p.n_slots) p.y[(size_t)sid * p.N + col] = (half_t)(v * s_tw[mb * 16 + m]);
+      float v[8];
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const int t = ww * 8 + awq_nibble_of_col(c);
+        v[c] = red[0][m][t * 16 + jj];
+        if (two) v[c] += red[1][m][t * 16 + jj];
       }
+      size_t orow = (size_t)(mb * 16 + m);
+      if (MOE) {
+        const int sid = s_sid[mb * 16 + m];
+        if (sid >= p.n_slots) continue;
+        const float tw = s_tw[mb * 16 + m];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) v[c] *= tw;
+        orow = (size_t)sid;
+      }
+      h8 o;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) o[c] = (half_t)v[c];
+      *reinterpret_cast<h8*>(p.y + orow * p.N + col) = o;
     }
   };
 
@@ -398,20 +413,28 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
   for (int mb = 0; mb < MB; ++mb) {
     const int rows = min(16, max(0, rows_total - 16 * mb));
     // ---- cross-wave sum in LDS: red[b][row][tile*16 + j] ----
+    // (rows past the block's last one are never read back)
     if (wave >= 2) {
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
+      for (int r = 0; r < 4; ++r)
+        if (4 * h + r < rows) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[wave - 2][4 * h + r][t * 16 + j] = w.acc[mb][t][r];
+          for (int t = 0; t < NT; ++t) red[wave - 2][4 * h + r][t * 16 + j] = w.acc[mb][t][r];
+        }
     }
     __syncthreads();
     if (wave < 2) {
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
+      for (int r = 0; r < 4; ++r)
+        if (4 * h + r < rows) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[wave][4 * h + r][t * 16 + j] += w.acc[mb][t][r];
+          for (int t = 0; t < NT; ++t) red[wave][4 * h + r][t * 16 + j] += w.acc[mb][t][r];
+        }
     }
     __syncthreads();
+#if defined(AWQMI_LAB_EPI) && AWQMI_LAB_EPI == 3
+    if (p.M != 12345) return;
+#endif
     if (split) {
       // fp32 partial tile of this workgroup.  Partials and the arrival counter go through
       // device-coherent accesses (they bypass the per-XCD L2 for other XCDs' data) instead of
@@ -419,10 +442,11 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
       // per workgroup, which costs far more than the few KB of partials.
       float* mine = p.part + (((size_t)sp * ntiles + tile) * MB + mb) * TILE_F;
       const int nelem = rows * (NT * 16);
-      for (int i = tid * 2; i < nelem; i += 512) {
+      for (int i = tid * 4; i < nelem; i += 1024) {
         const int m = i / (NT * 16), c = i % (NT * 16);
-        const f2 v = *reinterpret_cast<const f2*>(&red[0][m][c]) + *reinterpret_cast<const f2*>(&red[1][m][c]);
-        st_coherent(mine + i, v);
+        const f4 v = *reinterpret_cast<const f4*>(&red[0][m][c]) + *reinterpret_cast<const f4*>(&red[1][m][c]);
+        st_coherent(mine + i, f2{v[0], v[1]});
+        st_coherent(mine + i + 2, f2{v[2], v[3]});
       }
     } else {
       emit(mb, rows, true);
@@ -430,6 +454,9 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
     __syncthreads();
   }
   if (!split) return;
+#if defined(AWQMI_LAB_EPI) && AWQMI_LAB_EPI == 2
+  if (p.M != 12345) return;
+#endif
 
   // Ordering: every store of this workgroup has completed (vmcnt 0, then the barrier)
   // before its arrival is counted; whoever arrives last sums all partials in fixed order.
@@ -438,24 +465,53 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
   if (tid == 0) s_last = (atomicAdd(p.cnt + tile, 1) == p.split_k - 1);
   __syncthreads();
   if (!s_last) return;
+#if defined(AWQMI_LAB_EPI) && AWQMI_LAB_EPI == 1
+  if (p.M != 12345) { if (tid == 0) __hip_atomic_store(p.cnt + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); return; }
+#endif
   const size_t sstride = ntiles * MB * TILE_F;
+  // U pairs per thread x 8 parts per batch: 8 * U independent 8-byte loads in flight; parts
+  // are added in index order whatever the arrival order was.  Out-of-range slots read a valid
+  // address and are dropped by a select, so no load sits behind a branch.
+  auto finish = [&](auto u_tag, const float* base, int nelem) {
+    constexpr int U = decltype(u_tag)::value;
+    constexpr int SU = 8;
+    f2 v[U];
+    int idx[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      v[u] = f2{0.f, 0.f};
+      idx[u] = tid * 2 + 512 * u;
+    }
+    for (int s0 = 0; s0 < p.split_k; s0 += SU) {
+      f2 t[SU][U];
+#pragma unroll
+      for (int su = 0; su < SU; ++su) {
+        const int sidx = min(s0 + su, p.split_k - 1);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          t[su][u] = ld_coherent(base + (size_t)sidx * sstride + min(idx[u], nelem - 2));
+      }
+#pragma unroll
+      for (int su = 0; su < SU; ++su) {
+        const bool ok = s0 + su < p.split_k;
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] += ok ? t[su][u] : f2{0.f, 0.f};
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (idx[u] < nelem) *reinterpret_cast<f2*>(&red[0][idx[u] / (NT * 16)][idx[u] % (NT * 16)]) = v[u];
+  };
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int rows = min(16, max(0, rows_total - 16 * mb));
     const int nelem = rows * (NT * 16);
     const float* base = p.part + (tile * MB + mb) * TILE_F;
-    for (int i = tid * 2; i < nelem; i += 512) {
-      f2 v = {0.f, 0.f};
-      int s = 0;
-      for (; s + 8 <= p.split_k; s += 8) {   // eight independent loads in flight, fixed order
-        f2 t[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) t[u] = ld_coherent(base + (size_t)(s + u) * sstride + i);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) v += t[u];
-      }
-      for (; s < p.split_k; ++s) v += ld_coherent(base + (size_t)s * sstride + i);
-      *reinterpret_cast<f2*>(&red[0][i / (NT * 16)][i % (NT * 16)]) = v;
+    if (nelem > 0) {
+      if (nelem <= 512) finish(std::integral_constant<int, 1>{}, base, nelem);
+      else if (nelem <= 1024) finish(std::integral_constant<int, 2>{}, base, nelem);
+      else if (nelem <= 2048) finish(std::integral_constant<int, 4>{}, base, nelem);
+      else finish(std::integral_constant<int, 8>{}, base, nelem);
     }
     __syncthreads();
     emit(mb, rows, false);
