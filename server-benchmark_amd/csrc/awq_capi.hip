@@ -81,12 +81,12 @@ inline size_t gemv_partial_bytes(int N, int split, long long blocks_z, int tile_
   return (size_t)split * (size_t)blocks_z * tile_m * npad * sizeof(float);
 }
 
-template <int WPL, int MB, bool MOE>
+template <int WPL, int MB, bool MOE, int RING = 4>
 void launch_gemv(const GemvParams& p, dim3 grid, hipStream_t st) {
-  if (p.G == 32) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MB, MOE>), grid, dim3(256), 0, st, p);
-  else if (p.G == 64) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MB, MOE>), grid, dim3(256), 0, st, p);
-  else if (p.G == 128) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MB, MOE>), grid, dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MB, MOE>), grid, dim3(256), 0, st, p);
+  if (p.G == 32) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MB, MOE, RING>), grid, dim3(256), 0, st, p);
+  else if (p.G == 64) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MB, MOE, RING>), grid, dim3(256), 0, st, p);
+  else if (p.G == 128) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MB, MOE, RING>), grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MB, MOE, RING>), grid, dim3(256), 0, st, p);
 }
 
 // rows the skinny kernel takes in one awq_gemm call (passes of up to 32 rows)
@@ -326,22 +326,43 @@ int awqmi_moe_align(const int32_t* topk_ids, int n_slots, int E, int tile_m, int
   return launch_status();
 }
 
-static int moe_pick_split(int n_slots, int E, int K, int N, int G, int nblk, int ncb, int tile_m) {
+// sorted-token blocks a grouped launch covers: the align capacity, rounded up to whole groups
+static int moe_launch_blocks(int n_slots, int E, int tile_m) {
+  const int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, tile_m) / tile_m);
+  return (nblk + MOE_BLOCK_GROUP_MAX - 1) / MOE_BLOCK_GROUP_MAX * MOE_BLOCK_GROUP_MAX;
+}
+
+// Launch shape of a grouped GEMM, shared by the workspace query and the launch itself.
+struct MoePlan { int wpl, ncb, nblk, split; };
+static MoePlan moe_plan(int n_slots, int E, int K, int N, int tile_m, int split_req) {
+  MoePlan pl{};
+  const int NW = N / 8;
+  pl.wpl = gemv_wpl(N);
+  pl.ncb = (NW + 16 * pl.wpl - 1) / (16 * pl.wpl);
+  pl.nblk = moe_launch_blocks(n_slots, E, tile_m);
+  const int nchunks = K / 128;
   // blocks that will actually run: at most one per tile_m slots plus one per expert touched
   long long live = (n_slots + tile_m - 1) / tile_m;
   const long long touched = n_slots < E ? n_slots : E;
   if (live < touched) live = touched;
-  int s = pick_split_k(16, K, N, G, live);
-  if ((size_t)nblk * ncb * sizeof(int) > AWQMI_WS_COUNTER_BYTES) s = 1;
-  return s;
+  int s = split_req;
+  if (s <= 0) {
+    if (K % 128 != 0) {
+      s = 1;
+    } else {
+      s = pick_split_k(16, K, N, 128, live);
+    }
+    if ((size_t)pl.nblk * pl.ncb * sizeof(int) > AWQMI_WS_COUNTER_BYTES) s = 1;
+  }
+  if (s > nchunks) s = nchunks > 0 ? nchunks : 1;
+  pl.split = s;
+  return pl;
 }
 
 size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int split_k, int tile_m) {
-  if (n_slots <= 0 || E <= 0 || K <= 0 || N <= 0 || (tile_m != 16 && tile_m != 32)) return 0;
-  const int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, tile_m) / tile_m);
-  int s = split_k;
-  if (s <= 0) s = (K % 128 == 0) ? moe_pick_split(n_slots, E, K, N, 128, nblk, (N + 127) / 128, tile_m) : 1;
-  return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, s, nblk, tile_m);
+  if (n_slots <= 0 || E <= 0 || K <= 0 || N <= 0 || N % 8 != 0 || (tile_m != 16 && tile_m != 32)) return 0;
+  const MoePlan pl = moe_plan(n_slots, E, K, N, tile_m, split_k);
+  return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, pl.split, pl.nblk, tile_m);
 }
 
 int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
@@ -363,13 +384,9 @@ int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales
       !aligned16(y))
     return AWQMI_BAD_ALIGN;
   const int NW = N / 8;
-  const int wpl = gemv_wpl(N);
+  const MoePlan pl = moe_plan(n_slots, E, K, N, tile_m, split_k);
+  const int wpl = pl.wpl, ncb = pl.ncb, nblk = pl.nblk, split = pl.split;
   if (tile_m == 32 && wpl != 2) return AWQMI_BAD_SHAPE;   // 32-row blocks need N % 16 == 0
-  const int ncb = (NW + 16 * wpl - 1) / (16 * wpl);
-  const int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, tile_m) / tile_m);
-  int split = split_k > 0 ? split_k : moe_pick_split(n_slots, E, K, N, G, nblk, ncb, tile_m);
-  const int nchunks = K / 128;
-  if (split > nchunks) split = nchunks;
   if (split > 1) {
     if (!workspace) return AWQMI_NULL_POINTER;
     if (!aligned16(workspace)) return AWQMI_BAD_ALIGN;
@@ -391,10 +408,18 @@ int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales
   p.sorted_ids = sorted_token_ids; p.expert_ids = expert_ids; p.n_post_pad = num_tokens_post_padded;
   p.topk_w = topk_weights; p.n_slots = n_slots; p.a_row_div = a_row_div; p.tile_m = tile_m;
   p.w_stride = (long long)K * NW; p.s_stride = (long long)(K / G) * N; p.z_stride = (long long)(K / G) * NW;
-  const dim3 grid(ncb, split, nblk);
+  p.nblk = nblk;
+  const int variant = g_gemv_variant.load(std::memory_order_relaxed);
+  // group blocks by XCD once experts average two blocks or more
+  p.grp = (long long)n_slots >= 2LL * tile_m * E ? 8 : 1;
+  if (variant >= 0 && ((variant >> 2) & 7)) p.grp = 1 << (((variant >> 2) & 7) - 1);
+  // runs of grp slots, dealt to the 8 XCDs in turn; the last deal may be partial
+  const long long runs = (long long)(nblk / p.grp) * ncb * split;
+  const dim3 grid((unsigned)((runs + 7) / 8 * 8 * p.grp));
   hipStream_t st = (hipStream_t)stream;
   if (tile_m == 32) launch_gemv<2, 2, true>(p, grid, st);
-  else if (wpl == 2) launch_gemv<2, 1, true>(p, grid, st);
+  else if (wpl == 2 && variant >= 0 && (variant & 2)) launch_gemv<2, 1, true, 4>(p, grid, st);
+  else if (wpl == 2) launch_gemv<2, 1, true, 2>(p, grid, st);
   else launch_gemv<1, 1, true>(p, grid, st);
   return launch_status();
 }

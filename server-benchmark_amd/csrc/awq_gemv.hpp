@@ -39,10 +39,20 @@ struct GemvParams {
   int n_slots;
   int a_row_div;
   int tile_m;   // rows per sorted-token block: 16 * MB
+  int nblk;     // sorted-token blocks covered by the launch (a multiple of grp)
+  int grp;      // sorted-token blocks per XCD run
   long long w_stride, s_stride, z_stride;  // elements per expert
 };
 
 typedef float f2 __attribute__((ext_vector_type(2)));
+
+// Expert-grouped launches use a 1-D grid and place work by XCD (workgroup i runs on XCD
+// i % 8, each XCD has its own L2): grp consecutive sorted-token blocks -- mostly blocks of
+// one or two experts -- times one (column block, K part) form a run of consecutive slots on
+// ONE XCD, so the blocks that share an expert read its weights through the same L2 at about
+// the same time instead of fetching them once per XCD.  grp = 1 is the plain order (column
+// block fastest), used when few experts get more than one block.
+constexpr int MOE_BLOCK_GROUP_MAX = 16;
 
 // 8-byte device-coherent store / load (relaxed, agent scope)
 __device__ __forceinline__ void st_coherent(float* p, f2 v) {
@@ -67,9 +77,12 @@ struct WordVec<2> {
   static __device__ __forceinline__ uint32_t get(u2v v, int w) { return w ? v.y : v.x; }
 };
 
-// Per-wave main loop.  Ring of four 32-row steps in flight (4 x 8 rows x WPL words + the
-// matching 16-byte activation slices per lane); ring slot = step index mod 4, so a "chunk" is
-// four steps aligned to 128 rows and group boundaries fall on fixed slots.
+// Per-wave main loop.  Ring of RING 32-row steps in flight (RING x 8 rows x WPL words + the
+// matching 16-byte activation slices per lane); ring slot = step index mod RING with RING
+// dividing 4, so a "chunk" is four steps aligned to 128 rows and group boundaries fall on fixed
+// slots.  RING = 4 is the streaming configuration (one wave per SIMD, 16 KB in flight per wave);
+// RING = 2 fits two waves per SIMD, for launches made of many short workgroups whose start-up
+// and epilogue then overlap another workgroup's loads.
 //
 // Arithmetic.  A nibble left in place under the mask 0x000F000F (0x00F000F0) *is* the fp16
 // subnormal w * 2^-24 (w * 2^-20), and the matrix core takes subnormal fp16 inputs exactly,
@@ -82,7 +95,7 @@ struct WordVec<2> {
 //
 // MB row blocks of 16 share every B operand (MB = 2 serves up to 32 rows per pass with the
 // unpack work of one).  GMODE: 0 -> G = 32, 1 -> G = 64, 2 -> G = 128, 3 -> G = 128 * i.
-template <int WPL, int GMODE, int MB>
+template <int WPL, int GMODE, int MB, int RING = 4>
 struct GemvWave {
   static constexpr int NT = 8 * WPL;                                   // 16-column tiles per wave
   static constexpr int KSPG = GMODE == 0 ? 1 : (GMODE == 1 ? 2 : 4);  // group boundaries per chunk
@@ -95,13 +108,12 @@ struct GemvWave {
   const uint32_t* qz;        // lane's zero-word pointer (wc applied)
   int NW, N, kspg, ngroups;  // kspg: 32-row steps per quantisation group
 
-  qvec q[4][8];
-  u4v a[4][MB];
+  qvec q[RING][8];
+  u4v a[RING][MB];
   f4 acc[MB][NT];    // sum over finished groups of s * accg (still carrying 2^-e)
   f4 accg[MB][NT];   // current group
-  qvec znext;
+  qvec znext, zcur;
   u4v snext[WPL], scur[WPL];
-  uint32_t zb[NT];   // B operand word of the zero-point MFMA: (-z, -z) * 2^-e
   float xsum[MB];    // this lane's sum of x over the current group
   NibbleMasks nm;
 
@@ -133,15 +145,8 @@ struct GemvWave {
   // take over the prefetched group parameters
   __device__ __forceinline__ void adopt_group() {
 #pragma unroll
-    for (int w = 0; w < WPL; ++w) {
-      scur[w] = snext[w];
-      const uint32_t zw = WordVec<WPL>::get(znext, w);
-      uint32_t t;
-      t = byte_pair<0>(zw, zw); zb[w * 8 + 0] = (t & nm.lo) | 0x80008000u; zb[w * 8 + 1] = (t & nm.hi) | 0x80008000u;
-      t = byte_pair<1>(zw, zw); zb[w * 8 + 2] = (t & nm.lo) | 0x80008000u; zb[w * 8 + 3] = (t & nm.hi) | 0x80008000u;
-      t = byte_pair<2>(zw, zw); zb[w * 8 + 4] = (t & nm.lo) | 0x80008000u; zb[w * 8 + 5] = (t & nm.hi) | 0x80008000u;
-      t = byte_pair<3>(zw, zw); zb[w * 8 + 6] = (t & nm.lo) | 0x80008000u; zb[w * 8 + 7] = (t & nm.hi) | 0x80008000u;
-    }
+    for (int w = 0; w < WPL; ++w) scur[w] = snext[w];
+    zcur = znext;
   }
 
   template <int B>
@@ -194,6 +199,11 @@ struct GemvWave {
     }
   }
 
+  static __device__ __forceinline__ uint32_t zbyte(uint32_t zw, int b) {
+    return b == 0 ? byte_pair<0>(zw, zw) : b == 1 ? byte_pair<1>(zw, zw)
+         : b == 2 ? byte_pair<2>(zw, zw) : byte_pair<3>(zw, zw);
+  }
+
   // end of a group: zero-point MFMA, then acc += s * accg
   __device__ __forceinline__ void flush() {
 #ifdef AWQMI_LAB_NO_COMPUTE
@@ -209,9 +219,19 @@ struct GemvWave {
       const h2 xp01 = {x0, x1}, xp2 = {x2, (half_t)0.f};
       const h8 az = as_h8(u4v{as_u32(xp01), as_u32(xp2), 0u, 0u});
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        const h8 bz = as_h8(u4v{zb[t], zb[t] & 0x0000FFFFu, 0u, 0u});
-        accg[mb][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(az, bz, accg[mb][t], 0, 0, 0);
+      for (int w = 0; w < WPL; ++w) {
+        const uint32_t zw = WordVec<WPL>::get(zcur, w);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          // B operand word of the zero-point MFMA: (-z, -z) * 2^-e in k-slots 0, 1 and -z in 2
+          const uint32_t t = zbyte(zw, b);
+          const uint32_t zlo = (t & nm.lo) | 0x80008000u, zhi = (t & nm.hi) | 0x80008000u;
+          const int t0 = w * 8 + 2 * b;
+          accg[mb][t0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+              az, as_h8(u4v{zlo, zlo & 0x0000FFFFu, 0u, 0u}), accg[mb][t0], 0, 0, 0);
+          accg[mb][t0 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+              az, as_h8(u4v{zhi, zhi & 0x0000FFFFu, 0u, 0u}), accg[mb][t0 + 1], 0, 0, 0);
+        }
       }
 #pragma unroll
       for (int w = 0; w < WPL; ++w) {
@@ -251,14 +271,14 @@ struct GemvWave {
             xsum[mb] = 0.f;
           }
         }
-        compute(d, false);
+        compute(d % RING, false);
       } else {
-        compute(d, d % KSPG == 0);
+        compute(d % RING, d % KSPG == 0);
       }
       // pin the refill right behind its slot's compute: sunk to the end of the chunk the
       // four-deep ring degenerates into load-all / wait-all / compute-all
       __builtin_amdgcn_sched_barrier(0);
-      if (REFILL) issue(d, 4 * c + d + 4);
+      if (REFILL || d + RING < 4) issue(d % RING, 4 * c + d + RING);
       __builtin_amdgcn_sched_barrier(0);
       if (GMODE != 3 && (d + 1) % KSPG == 0) flush();
     }
@@ -279,7 +299,7 @@ struct GemvWave {
     nm.init();
     load_group(clamp_group(4 * c_begin));
 #pragma unroll
-    for (int d = 0; d < 4; ++d) issue(d, 4 * c_begin + d);
+    for (int d = 0; d < RING; ++d) issue(d, 4 * c_begin + d);
     int c = c_begin;
     for (; c + 1 < c_end; ++c) chunk<true>(c, c_begin, c_end);
     chunk<false>(c, c_begin, c_end);
@@ -291,8 +311,8 @@ struct GemvWave {
   }
 };
 
-template <int WPL, int GMODE, int MB, bool MOE>
-__global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kernel(const GemvParams p) {
+template <int WPL, int GMODE, int MB, bool MOE, int RING = 4>
+__global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
   constexpr int NT = 8 * WPL;
   constexpr int CB = 128 * WPL;
   constexpr int RS = NT * 16 + 4;  // LDS row stride in floats: 4h rows land 16 banks apart
@@ -304,14 +324,21 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
   __shared__ int s_rows;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, h = lane >> 4;
-  const int cb = blockIdx.x, sp = blockIdx.y;
+  int cb = blockIdx.x, sp = blockIdx.y;
   int blk = 0;
   const uint32_t* qw = p.qw;
   const half_t* sc = p.sc;
   const uint32_t* qz = p.qz;
   if (MOE) {
-    blk = blockIdx.z;
-    if (blk * TM >= *p.n_post_pad) return;
+    const int B = p.grp;
+    const int lin = blockIdx.x, xcd = lin & 7, slot = lin >> 3;
+    const int g = (slot / B) * 8 + xcd;            // run index: (block group, column block, part)
+    const int ncbs = p.ncb * p.split_k;
+    const int bg = g / ncbs, cbs = g % ncbs;
+    blk = bg * B + slot % B;
+    cb = cbs / p.split_k;
+    sp = cbs % p.split_k;
+    if (blk >= p.nblk || blk * TM >= *p.n_post_pad) return;
     const int e = p.expert_ids[blk];
     qw += (size_t)e * p.w_stride;
     sc += (size_t)e * p.s_stride;
@@ -336,7 +363,7 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
   int wc = cb * (16 * WPL) + WPL * j;
   if (wc >= p.NW) wc = 0;
 
-  GemvWave<WPL, GMODE, MB> w;
+  GemvWave<WPL, GMODE, MB, RING> w;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int r = mb * 16 + j;
@@ -373,7 +400,7 @@ __global__ __launch_bounds__(256, AWQMI_GEMV_WAVES_PER_SIMD) void awq_gemv_kerne
 
   const int rows_total = MOE ? s_rows : p.M;
   const size_t tile = (size_t)blk * p.ncb + cb;
-  const size_t ntiles = (size_t)(MOE ? gridDim.z : 1) * p.ncb;
+  const size_t ntiles = (size_t)(MOE ? p.nblk : 1) * p.ncb;
   constexpr int TILE_F = 16 * NT * 16;   // floats per partial tile (one row block)
   const bool split = p.split_k > 1;
 
