@@ -341,17 +341,40 @@ def main():
                 ym = sba.fused_moe_awq(xm, w13, w2, lg, topk, True)
             b.record()
             torch.cuda.synchronize()
+            us_eager = a.elapsed_time(b) * 1e3 / n_it
+            # the same call replayed from a HIP graph (how a serving engine runs decode steps)
+            gs = torch.cuda.Stream()
+            gs.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(gs):
+                ym = sba.fused_moe_awq(xm, w13, w2, lg, topk, True)      # sizes this stream's workspace
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=gs):
+                    yg = sba.fused_moe_awq(xm, w13, w2, lg, topk, True)
+                for _ in range(3):
+                    graph.replay()
+                torch.cuda.synchronize()
+                a.record()
+                for _ in range(n_it):
+                    graph.replay()
+                b.record()
+                torch.cuda.synchronize()
+            torch.cuda.current_stream().wait_stream(gs)
             us = a.elapsed_time(b) * 1e3 / n_it
+            if not torch.equal(yg, ym):
+                raise RuntimeError(f"MoE block T={T}: graph replay differs from the eager call")
+            del graph
             nbytes = workloads.moe_bytes(distinct, T, H, I, G)
             fl = workloads.moe_flops(T, topk, H, I)
-            mo.append({"T": T, "distinct_experts": distinct, "us": round(us, 1),
+            mo.append({"T": T, "distinct_experts": distinct, "us": round(us, 1), "us_eager_call": round(us_eager, 1),
                        "GBps": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                        "TFLOPs": round(fl / us / 1e6, 2)})
             if args.detail:
-                log(f"   moe T={T:4d} experts hit {distinct:3d}  {us:9.1f} us  {nbytes / us / 1e3:8.1f} GB/s")
+                log(f"   moe T={T:4d} experts hit {distinct:3d}  {us:9.1f} us (eager call {us_eager:6.1f})  "
+                    f"{nbytes / us / 1e3:8.1f} GB/s")
         out["moe"] = {"workload": "Qwen3-30B-A3B MoE block: route + align + grouped w13 GEMM + SiLU*up + grouped w2 "
                                   "GEMM + slot sum, 128 experts, top-8, hidden 2048, inter 768 (whole block per call, "
-                                  "weights not rotated: cache-warm for small T)",
+                                  "replayed from a HIP graph; weights not rotated: cache-warm for small T)",
                       "points": mo}
         del w13, w2
 

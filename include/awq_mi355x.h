@@ -125,6 +125,25 @@ int awqmi_silu_and_mul_f16(const void* in_f16, void* out_f16, int rows, int inte
 /* out[t, :] = sum over the topk slot rows in[t*topk + j, :], fp32 sum, fp16 out. */
 int awqmi_moe_sum_f16(const void* in_f16, void* out_f16, int T, int topk, int H, void* stream);
 
+/* One whole AWQ MoE block in one call: softmax + top-k routing, align, grouped w13 GEMM,
+ * SiLU(gate) * up, grouped w2 GEMM scaled by the routing weights, sum over each token's
+ * slots.  Replaces the sequence fused_topk -> moe_align_block_size -> fused_experts that
+ * the AWQ MoE method runs (vLLM model_executor/layers/quantization/awq.py, AWQMoEMethod.apply ->
+ * layers/fused_moe/fused_moe.py fused_experts; the harness reaches it through
+ * docker-compose.vllm.yml:13-16 with an AWQ MoE checkpoint).
+ *   hidden fp16 [T, H]; router_logits fp32 [T, E]; out fp16 [T, H]
+ *   w13: qweight int32 [E, H, 2*inter/8], scales fp16 [E, H/G, 2*inter], qzeros int32 [E, H/G, 2*inter/8]
+ *        (columns [gate | up]);  w2: [E, inter, H/8], [E, inter/G, H], [E, inter/G, H/8]
+ * Every intermediate lives in the workspace (awqmi_fused_moe_workspace_bytes), which must be
+ * zero-initialised once; the call itself allocates nothing and is safe to capture in a HIP
+ * graph.  H and inter must be multiples of 128 with group in {32, 64, 128 * i}. */
+size_t awqmi_fused_moe_workspace_bytes(int T, int H, int inter, int E, int topk);
+int awqmi_fused_moe_f16(const void* hidden_f16, const float* router_logits, const int32_t* w13_qweight,
+                        const void* w13_scales_f16, const int32_t* w13_qzeros,
+                        const int32_t* w2_qweight, const void* w2_scales_f16, const int32_t* w2_qzeros,
+                        void* out_f16, int T, int H, int inter, int E, int topk, int group,
+                        int renormalize, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Development hook: choose among equivalent kernel variants of the skinny GEMM
  * (-1 = library default).  Returns the previous value.  Not part of the stable surface. */
 int awqmi_set_gemv_variant(int variant);

@@ -446,4 +446,78 @@ int awqmi_moe_sum_f16(const void* in, void* out, int T, int topk, int H, void* s
   return launch_status();
 }
 
+namespace {
+// workspace carve-up of the fused MoE block; every piece starts 256-byte aligned
+struct FusedMoeLayout {
+  size_t gemm_ws, ids, wts, sorted, experts, npp, h13, act, o, total;
+  size_t gemm_ws_bytes;
+  int n_slots, cap;
+};
+FusedMoeLayout fused_moe_layout(int T, int H, int inter, int E, int topk) {
+  FusedMoeLayout L{};
+  auto up = [](size_t v) { return (v + 255) / 256 * 256; };
+  L.n_slots = T * topk;
+  L.cap = (int)awqmi_moe_align_capacity(L.n_slots, E, 16);
+  const size_t g1 = awqmi_moe_gemm_workspace_bytes(L.n_slots, E, H, 2 * inter, 0, 16);
+  const size_t g2 = awqmi_moe_gemm_workspace_bytes(L.n_slots, E, inter, H, 0, 16);
+  L.gemm_ws_bytes = g1 > g2 ? g1 : g2;
+  size_t off = 0;
+  L.gemm_ws = off; off += up(L.gemm_ws_bytes);
+  L.ids = off;     off += up((size_t)L.n_slots * 4);
+  L.wts = off;     off += up((size_t)L.n_slots * 4);
+  L.sorted = off;  off += up((size_t)L.cap * 4);
+  L.experts = off; off += up((size_t)(L.cap / 16) * 4);
+  L.npp = off;     off += 256;
+  L.h13 = off;     off += up((size_t)L.n_slots * 2 * inter * 2);
+  L.act = off;     off += up((size_t)L.n_slots * inter * 2);
+  L.o = off;       off += up((size_t)L.n_slots * H * 2);
+  L.total = off;
+  return L;
+}
+}  // namespace
+
+size_t awqmi_fused_moe_workspace_bytes(int T, int H, int inter, int E, int topk) {
+  if (T <= 0 || H <= 0 || inter <= 0 || E <= 0 || topk <= 0 || H % 8 != 0 || inter % 8 != 0) return 0;
+  if ((long long)T * topk > (1LL << 30)) return 0;
+  return fused_moe_layout(T, H, inter, E, topk).total;
+}
+
+int awqmi_fused_moe_f16(const void* hidden, const float* router_logits, const int32_t* w13_q,
+                        const void* w13_s, const int32_t* w13_z, const int32_t* w2_q, const void* w2_s,
+                        const int32_t* w2_z, void* out, int T, int H, int inter, int E, int topk,
+                        int group, int renormalize, void* workspace, size_t workspace_bytes,
+                        void* stream) {
+  if (!hidden || !router_logits || !w13_q || !w13_s || !w13_z || !w2_q || !w2_s || !w2_z || !out ||
+      !workspace)
+    return AWQMI_NULL_POINTER;
+  if (T <= 0 || H <= 0 || inter <= 0 || E <= 0 || H % 8 != 0 || inter % 8 != 0) return AWQMI_BAD_SHAPE;
+  if (topk <= 0 || topk > E || topk > 64 || E > AWQMI_MAX_EXPERTS || (long long)T * topk > (1LL << 30))
+    return AWQMI_BAD_ARGUMENT;
+  if (!aligned16(workspace)) return AWQMI_BAD_ALIGN;
+  const FusedMoeLayout L = fused_moe_layout(T, H, inter, E, topk);
+  if (workspace_bytes < L.total) return AWQMI_WORKSPACE_TOO_SMALL;
+  char* ws = static_cast<char*>(workspace);
+  int32_t* ids = reinterpret_cast<int32_t*>(ws + L.ids);
+  float* wts = reinterpret_cast<float*>(ws + L.wts);
+  int32_t* sorted = reinterpret_cast<int32_t*>(ws + L.sorted);
+  int32_t* experts = reinterpret_cast<int32_t*>(ws + L.experts);
+  int32_t* npp = reinterpret_cast<int32_t*>(ws + L.npp);
+  void* h13 = ws + L.h13;
+  void* act = ws + L.act;
+  void* o = ws + L.o;
+  int st = awqmi_moe_topk_softmax_f32(router_logits, T, E, topk, renormalize, ids, wts, stream);
+  if (st) return st;
+  st = awqmi_moe_align(ids, L.n_slots, E, 16, sorted, experts, npp, stream);
+  if (st) return st;
+  st = awqmi_moe_gemm_f16(hidden, w13_q, w13_s, w13_z, h13, sorted, experts, npp, nullptr, L.n_slots, topk,
+                          16, E, H, 2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream);
+  if (st) return st;
+  st = awqmi_silu_and_mul_f16(h13, act, L.n_slots, inter, stream);
+  if (st) return st;
+  st = awqmi_moe_gemm_f16(act, w2_q, w2_s, w2_z, o, sorted, experts, npp, wts, L.n_slots, 1, 16, E, inter, H,
+                          group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream);
+  if (st) return st;
+  return awqmi_moe_sum_f16(o, out, T, topk, H, stream);
+}
+
 }  // extern "C"

@@ -217,7 +217,36 @@ def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Ten
                   renormalize: bool = True, block_size: int | None = None) -> torch.Tensor:
     """One AWQ MoE block: route -> align -> grouped GEMM (w13) -> SiLU*up -> grouped GEMM (w2,
     scaled by the routing weight) -> sum over slots.  w13 / w2 are (qweight, scales, qzeros)
-    with a leading expert dimension; w13 columns are [gate | up]."""
+    with a leading expert dimension; w13 columns are [gate | up].  With block_size left at
+    None the block runs as one library call; a block size selects the step-by-step path."""
+    _need(hidden_states, "hidden_states", torch.float16, 2)
+    T, H = hidden_states.shape
+    E = w13[0].shape[0]
+    if block_size is None:
+        # the whole block in one library call, intermediates in the workspace
+        for i, (t, dt) in enumerate(zip(tuple(w13) + tuple(w2), (torch.int32, torch.float16, torch.int32) * 2)):
+            _need(t, f"w13/w2[{i}]", dt, 3)
+        K1, N1, G1 = _awq_shapes(*w13, lead=1)
+        K2, N2, G2 = _awq_shapes(*w2, lead=1)
+        inter = N1 // 2
+        if K1 != H or N2 != H or K2 != inter or N1 != 2 * inter or G1 != G2 or w2[0].shape[0] != E:
+            raise ValueError(f"w13 [{K1}, {N1}] / w2 [{K2}, {N2}] do not fit hidden {H}")
+        lg = gating_output
+        if lg.dtype != torch.float32 or not lg.is_contiguous():
+            lg = lg.float().contiguous()
+        _need(lg, "gating_output", torch.float32, 2)
+        if tuple(lg.shape) != (T, E):
+            raise ValueError(f"gating_output shape {tuple(lg.shape)} != ({T}, {E})")
+        lib = _lib.load()
+        nbytes = lib.awqmi_fused_moe_workspace_bytes(T, H, inter, E, topk)
+        ws = get_workspace(hidden_states.device, nbytes)
+        out = torch.empty((T, H), dtype=torch.float16, device=hidden_states.device)
+        st = lib.awqmi_fused_moe_f16(hidden_states.data_ptr(), lg.data_ptr(), w13[0].data_ptr(), w13[1].data_ptr(),
+                                     w13[2].data_ptr(), w2[0].data_ptr(), w2[1].data_ptr(), w2[2].data_ptr(),
+                                     out.data_ptr(), T, H, inter, E, topk, G1, int(renormalize), ws.data_ptr(),
+                                     ws.numel(), _stream_ptr(hidden_states.device))
+        _lib.check(st, "fused_moe_awq")
+        return out
     T = hidden_states.shape[0]
     E = w13[0].shape[0]
     topk_w, topk_ids = topk_softmax(gating_output.float().contiguous(), topk, renormalize)

@@ -127,3 +127,36 @@ def test_moe_qwen3_shapes_vs_dense_expert_path(sba, gpu, T):
     err = awq_ref.rel_frobenius(y.cpu().numpy(), ref.cpu().numpy())
     print(f"[moe T={T} vs dense experts] rel_fro={err:.2e}", flush=True)
     assert err <= TOL
+
+
+@pytest.mark.parametrize("T", [1, 7, 64])
+def test_fused_call_equals_step_by_step(sba, gpu, T):
+    """The one-call block and the six separate calls run the same kernels on the same data:
+    bit-identical outputs, also on a second call that reuses the workspace."""
+    c = sba.workloads.make_moe_case(T, 512, 16, 4, 256, 128, seed=7 + T).to(gpu)
+    step = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 4, True, block_size=16)
+    for _ in range(2):
+        one = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 4, True)
+        assert torch.equal(one, step)
+
+
+def test_fused_call_graph_replay(sba, gpu):
+    """Captured once, replayed with eager work in between: every replay equals the eager result."""
+    c = sba.workloads.make_moe_case(16, 2048, 128, 8, 768, 128, seed=3).to(gpu)
+    eager = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 8, True)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 8, True)   # sizes this stream's workspace
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            y = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 8, True)
+        for _ in range(3):
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, eager)
+            y.zero_()
+            sba.awq_gemm(c.x, c.w13[0][0], c.w13[1][0], c.w13[2][0], 0)   # unrelated eager work
+            torch.cuda.synchronize()
+    torch.cuda.current_stream().wait_stream(s)

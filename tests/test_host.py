@@ -65,6 +65,25 @@ def test_validation_happens_before_any_launch(lib):
                                   0, 0, 0, 0) == 7
     assert lib.awqmi_silu_and_mul_f16(fake, fake, 4, 12, 0) == 1
     assert lib.awqmi_moe_sum_f16(fake, fake, 4, 2, 12, 0) == 1
+    # whole-block MoE call: null operand, top-k beyond E, short workspace
+    ok = [fake] * 9
+    assert lib.awqmi_fused_moe_f16(*ok[:8], 0, 4, 256, 128, 8, 2, 128, 1, fake, 1 << 30, 0) == 6
+    assert lib.awqmi_fused_moe_f16(*ok, 4, 256, 128, 8, 9, 128, 1, fake, 1 << 30, 0) == 7
+    assert lib.awqmi_fused_moe_f16(*ok, 4, 256, 128, 8, 2, 128, 1, fake, 1024, 0) == 3
+    assert lib.awqmi_fused_moe_f16(*ok, 4, 250, 128, 8, 2, 128, 1, fake, 1 << 30, 0) == 1
+
+
+def test_fused_moe_workspace_covers_every_intermediate(lib):
+    T, H, I, E, topk = 16, 2048, 768, 128, 8
+    n = T * topk
+    total = lib.awqmi_fused_moe_workspace_bytes(T, H, I, E, topk)
+    g = max(lib.awqmi_moe_gemm_workspace_bytes(n, E, H, 2 * I, 0, 16),
+            lib.awqmi_moe_gemm_workspace_bytes(n, E, I, H, 0, 16))
+    cap = lib.awqmi_moe_align_capacity(n, E, 16)
+    payload = g + 2 * n * 4 + cap * 4 + cap // 16 * 4 + 4 + n * 2 * I * 2 + n * I * 2 + n * H * 2
+    assert payload <= total <= payload + 9 * 256
+    assert lib.awqmi_fused_moe_workspace_bytes(0, H, I, E, topk) == 0
+    assert lib.awqmi_fused_moe_workspace_bytes(T, H, 100, E, topk) == 0
 
 
 def test_workspace_and_split_k_queries(lib):
