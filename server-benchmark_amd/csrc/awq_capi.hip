@@ -92,6 +92,13 @@ void launch_gemv(const GemvParams& p, dim3 grid, hipStream_t st) {
 // rows the skinny kernel takes in one awq_gemm call (passes of up to 32 rows)
 constexpr int SKINNY_MAX_M = 64;
 
+// Between 33 and 64 rows two skinny passes compete with the 128-row MFMA tile: the MFMA
+// kernel wins while its tiles (times the K split) fit one round of workgroups, the skinny
+// kernel wins on very wide layers, where the MFMA tiles alone fill the chip.
+inline bool skinny_rows(int M, int N) {
+  return M <= 32 || (M <= SKINNY_MAX_M && (N + 255) / 256 > 128);
+}
+
 // Work split of the MFMA kernel: whole rounds of 256 tiles run one workgroup per tile; a
 // last round of fewer than 129 tiles (and any launch that small) is split in K over
 // floor(256 / tiles) workgroups per tile (at most 8, at least 8 k-tiles each).
@@ -166,19 +173,21 @@ int awqmi_dequantize_f16(const int32_t* qweight, const void* scales, const int32
 int awqmi_gemm_auto_split_k(int M, int K, int N, int group) {
   const int G = norm_group(K, group);
   if (check_awq_shape(K, N, G) != AWQMI_OK || M <= 0) return 1;
-  if (M > SKINNY_MAX_M || !gemv_tiled_ok(K, G)) return 1;
+  if (!skinny_rows(M, N) || !gemv_tiled_ok(K, G)) return 1;
   return pick_split_k(M, K, N, G, 1);
 }
 
 size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
   if (M <= 0 || K <= 0 || N <= 0) return 0;
-  if (M > SKINNY_MAX_M) {
-    if (K % PF_BK != 0) return AWQMI_WS_COUNTER_BYTES;
-    return AWQMI_WS_COUNTER_BYTES + plan_mfma(M, K, N).part_bytes;
+  // the group size decides between the kernels for some shapes, so cover both
+  size_t mfma = 0, skinny = 0;
+  if (M > 16 && K % PF_BK == 0) mfma = plan_mfma(M, K, N).part_bytes;
+  if (M <= SKINNY_MAX_M) {
+    int s = split_k;
+    if (s <= 0) s = (K % 128 == 0) ? pick_split_k(M, K, N, 128, 1) : 1;
+    skinny = gemv_partial_bytes(N, s, 1, 32);
   }
-  int s = split_k;
-  if (s <= 0) s = (K % 128 == 0) ? pick_split_k(M, K, N, 128, 1) : 1;
-  return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, s, 1, 32);
+  return AWQMI_WS_COUNTER_BYTES + (mfma > skinny ? mfma : skinny);
 }
 
 int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
@@ -201,7 +210,11 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   half_t* yy = reinterpret_cast<half_t*>(y);
 
   const int wpl = gemv_wpl(N);
-  if (gemv_tiled_ok(K, G) && (M <= 16 || (M <= SKINNY_MAX_M && wpl == 2))) {
+  const bool mfma_ok = K % PF_BK == 0 && (((G & (G - 1)) == 0 && G >= 8) || G % 64 == 0) &&
+                       (size_t)M * K * 2 < (1ull << 32) && (size_t)K * NW * 4 < (1ull << 32) &&
+                       (size_t)(K / G) * N * 2 < (1ull << 32);
+  if (gemv_tiled_ok(K, G) &&
+      (M <= 16 || (M <= SKINNY_MAX_M && wpl == 2 && (skinny_rows(M, N) || !mfma_ok)))) {
     int split = split_k > 0 ? split_k : pick_split_k(M, K, N, G, 1);
     const int nchunks = K / 128;
     if (split > nchunks) split = nchunks;
@@ -241,12 +254,14 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   if (K % PF_BK == 0 && (pow2g || G % 64 == 0) && small) {
     static std::atomic<bool> attr_set{false};
     if (!attr_set.load(std::memory_order_acquire)) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, PF_LDS_BYTES);
-      if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, PF_LDS_BYTES);
-      if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
+      const void* fns[4] = {reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 4>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 2>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 2>)};
+      for (const void* fn : fns) {
+        const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, PF_LDS_BYTES);
+        if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
+      }
       attr_set.store(true, std::memory_order_release);
     }
     MfmaGemmParams p{};
@@ -254,7 +269,9 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     p.M = M; p.K = K; p.N = N; p.NW = NW; p.G = G;
     p.gshift = 0;
     if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
-    p.mt = (M + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
+    // at most 128 rows: one row of 128-row tiles (half the MFMA work of a padded 256-row tile)
+    const bool half_tile = M <= 128;
+    p.mt = half_tile ? 1 : (M + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
     p.total = p.mt * p.nt;
     MfmaPlan pl = plan_mfma(M, K, N);
     // the K split needs the caller's workspace (counters + partial tiles); without it every
@@ -264,14 +281,23 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
       pl = MfmaPlan{p.total, 0, 1, 0};
     p.dp_tiles = pl.dp_tiles; p.sk_tiles = pl.sk_tiles; p.sk_split = pl.sk_split;
     p.per_xcd = (pl.dp_tiles + 7) / 8;
-    p.sk_cnt = reinterpret_cast<int*>(workspace);
     p.sk_part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
                           : nullptr;
     const dim3 grid(p.per_xcd * 8 + p.sk_tiles * p.sk_split);
-    if (pow2g)
-      hipLaunchKernelGGL(awq_gemm_mfma_kernel<true>, grid, dim3(256), PF_LDS_BYTES, st, p);
+    if (half_tile && pow2g)
+      hipLaunchKernelGGL((awq_gemm_mfma_kernel<true, 2>), grid, dim3(256), PF_LDS_BYTES, st, p);
+    else if (half_tile)
+      hipLaunchKernelGGL((awq_gemm_mfma_kernel<false, 2>), grid, dim3(256), PF_LDS_BYTES, st, p);
+    else if (pow2g)
+      hipLaunchKernelGGL((awq_gemm_mfma_kernel<true, 4>), grid, dim3(256), PF_LDS_BYTES, st, p);
     else
-      hipLaunchKernelGGL(awq_gemm_mfma_kernel<false>, grid, dim3(256), PF_LDS_BYTES, st, p);
+      hipLaunchKernelGGL((awq_gemm_mfma_kernel<false, 4>), grid, dim3(256), PF_LDS_BYTES, st, p);
+    if (p.sk_tiles > 0) {
+      if (half_tile)
+        hipLaunchKernelGGL(awq_gemm_mfma_reduce_kernel<2>, dim3(p.sk_tiles * 8), dim3(256), 0, st, p);
+      else
+        hipLaunchKernelGGL(awq_gemm_mfma_reduce_kernel<4>, dim3(p.sk_tiles * 16), dim3(256), 0, st, p);
+    }
     return launch_status();
   }
 

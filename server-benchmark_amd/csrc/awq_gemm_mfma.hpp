@@ -40,11 +40,11 @@ struct MfmaGemmParams {
   // Work split.  Tiles [0, dp_tiles) run one workgroup per tile over all of K (launch ids
   // [0, 8 * per_xcd)).  The remaining sk_tiles tiles (a last round that would leave most CUs
   // idle) are split in K over sk_split workgroups each (launch ids from 8 * per_xcd on,
-  // tile-major); the contributor that arrives last sums the fp32 partial tiles in the
-  // workspace in fixed order and writes the result.
+  // tile-major) and leave fp32 partial tiles in the workspace; a second, short kernel on the
+  // same stream sums them in part order and writes fp16 (a single finishing workgroup per
+  // tile would have to pull sk_split x 256 KiB by itself, which took longer than the GEMM).
   int dp_tiles, sk_tiles, sk_split;
   float* sk_part;   // [sk_tiles][sk_split][256 * 256] fp32
-  int* sk_cnt;      // [sk_tiles] arrival counters (zero before and after the launch)
 };
 
 constexpr int PF_SK_SLOT_FLOATS = 256 * 256;
@@ -68,8 +68,14 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* base, size
 
 // POW2G: G is a power of two (group index by shift, any G >= 8); otherwise G % 64 == 0 and
 // a k-tile lies inside one group (group index on the scalar unit).
-template <bool POW2G>
+//
+// MI = 32-row MFMA tiles per wave along M: 4 gives the 256-row workgroup tile; 2 gives a
+// 128-row tile (each wave 64 x 128) for launches of at most 128 rows, which would leave half
+// of a 256-row tile multiplying padding.
+template <bool POW2G, int MI = 4>
 __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmParams p) {
+  constexpr int BM = 64 * MI;      // workgroup tile rows
+  constexpr int AL = 2 * MI;       // 16-byte X loads per thread and k-tile
   extern __shared__ __align__(16) unsigned char smem_raw[];
   unsigned char* const As = smem_raw;                        // [2][256][128 B]
   unsigned char* const Bs = smem_raw + 2 * PF_TILE_BYTES;    // [2][256][128 B]
@@ -77,7 +83,6 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int id = blockIdx.x;
   const int KT = p.K / PF_BK;
-  __shared__ int s_last;
   int nid, kb = 0, ke = KT, part = -1;
   if (id < 8 * p.per_xcd) {
     nid = (id & 7) * p.per_xcd + (id >> 3);
@@ -94,8 +99,8 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   const int gm = min(p.mt - first_m, 8);
   const int mt_i = first_m + (nid % gsize) % gm;
   const int nt_i = (nid % gsize) / gm;
-  const int m0 = mt_i * PF_BM, n0 = nt_i * PF_BN;
-  const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
+  const int m0 = mt_i * BM, n0 = nt_i * PF_BN;
+  const int wm = (wave >> 1) * (32 * MI), wn = (wave & 1) * 128;
 
   const __amdgpu_buffer_rsrc_t rx = pf_rsrc(p.x, (size_t)p.M * p.K * 2);
   const __amdgpu_buffer_rsrc_t rw = pf_rsrc(p.qw, (size_t)p.K * p.NW * 4);
@@ -106,10 +111,10 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   // X tile: thread (a_row + 32 i, a_seg) moves 16 bytes; rows past M re-read row M - 1 (their
   // outputs are never stored), so no load sits behind a branch.
   const int a_row = tid >> 3, a_seg = tid & 7;
-  uint32_t a_off[8];
-  int a_dst[8];
+  uint32_t a_off[AL];
+  int a_dst[AL];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < AL; ++i) {
     const int r = a_row + 32 * i;
     const int gr = min(m0 + r, p.M - 1);
     a_off[i] = (uint32_t)(((size_t)gr * p.K + 8 * a_seg) * 2);
@@ -133,9 +138,9 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
 #pragma unroll
   for (int c = 0; c < 4; ++c) f_off[c] = fi * PF_ROW_BYTES + ((fu ^ (2 * c)) << 4);
 
-  f16v acc[4][4];
+  f16v acc[MI][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -143,14 +148,14 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
 
   NibbleMasks nm;
   nm.init();
-  u4v areg[8];          // X tile in flight
+  u4v areg[AL];         // X tile in flight
   uint32_t wreg[2][8];  // two W tiles in flight (parity of the k-tile)
   uint32_t zreg[2];
   u4v sreg[2];
   auto gload_a = [&](int kt) {
     const int so = kt * (PF_BK * 2);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, a_off[i], so, 0);
+    for (int i = 0; i < AL; ++i) areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, a_off[i], so, 0);
   };
   auto gload_w = [&](int kt, int set) {
     const uint32_t so = (uint32_t)kt * PF_BK * row_b;
@@ -170,7 +175,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   auto store_a = [&](int buf) {
     unsigned char* as = As + buf * PF_TILE_BYTES;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u4v*>(as + a_dst[i]) = areg[i];
+    for (int i = 0; i < AL; ++i) *reinterpret_cast<u4v*>(as + a_dst[i]) = areg[i];
   };
   // dequantise byte B (two columns x eight rows) of W register set `set` into buffer `buf`
   auto dq_byte = [&](int buf, int set, auto BTAG) {
@@ -195,12 +200,12 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
     *reinterpret_cast<u4v*>(bs + b_base + ch * PF_ROW_BYTES + ((b_t ^ ch) << 4)) = hi;
   };
 
-  h8 af[2][4], bf[2][4];   // fragments of two 16-wide k-steps
+  h8 af[2][MI], bf[2][4];  // fragments of two 16-wide k-steps
   auto load_frags = [&](int buf, int ks, int fs) {
     const unsigned char* as = As + buf * PF_TILE_BYTES + wm * PF_ROW_BYTES;
     const unsigned char* bs = Bs + buf * PF_TILE_BYTES + wn * PF_ROW_BYTES;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MI; ++i)
       af[fs][i] = *reinterpret_cast<const h8*>(as + 32 * i * PF_ROW_BYTES + f_off[ks ^ (2 * (i & 1))]);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -208,7 +213,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   };
   auto mfma_step = [&](int fs) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[fs][i], bf[fs][j], acc[i][j], 0, 0, 0);
@@ -222,7 +227,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
     constexpr int valu = decltype(VALU)::value, dsr = decltype(DSR)::value;
     constexpr int dsw = decltype(DSW)::value, vm = decltype(VM)::value;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < 2 * MI; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       if (dsr) __builtin_amdgcn_sched_group_barrier(0x100, dsr, 0);
       if (vm) __builtin_amdgcn_sched_group_barrier(0x020, vm, 0);
@@ -236,8 +241,12 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
-  using I6 = std::integral_constant<int, 6>;
-  using I12 = std::integral_constant<int, 12>;
+  // per-MFMA-pair shares; the 128-row tile has half the MFMAs per phase for the same W work
+  using VA = std::integral_constant<int, MI == 4 ? 6 : 12>;    // dequant VALU, phases 1 and 2
+  using VB = std::integral_constant<int, MI == 4 ? 12 : 24>;   // phase 3
+  using DR = std::integral_constant<int, MI == 4 ? 1 : 2>;     // fragment reads
+  using DW1 = std::integral_constant<int, MI == 4 ? 1 : 3>;    // LDS writes, phase 1 (X tile + byte 0)
+  using VM1 = std::integral_constant<int, MI == 4 ? 2 : 3>;    // W / zero / scale loads, phase 1
 
   // One k-tile, PAR = kt & 1.  On entry: LDS buffer PAR holds tile kt and fragment set 0 its
   // first k-step; areg and W set PAR^1 hold tile kt + 1; W set PAR is free.  Tiles past the
@@ -252,7 +261,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
     store_a(PAR ^ 1);
     gload_w(kt2, PAR);
     dq_byte(PAR ^ 1, PAR ^ 1, I0{});
-    phase_schedule(I6{}, I1{}, I1{}, I2{});
+    phase_schedule(VA{}, DR{}, DW1{}, VM1{});
     __builtin_amdgcn_sched_barrier(0);
 
     // phase 2: X(kt+2) -> registers, byte 1 of W(kt+1)
@@ -260,7 +269,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
     load_frags(PAR, 2, 0);
     gload_a(kt2);
     dq_byte(PAR ^ 1, PAR ^ 1, I1{});
-    phase_schedule(I6{}, I1{}, I1{}, I1{});
+    phase_schedule(VA{}, DR{}, I1{}, I1{});
     __builtin_amdgcn_sched_barrier(0);
 
     // phase 3: bytes 2 and 3 of W(kt+1)
@@ -268,7 +277,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
     load_frags(PAR, 3, 1);
     dq_byte(PAR ^ 1, PAR ^ 1, I2{});
     dq_byte(PAR ^ 1, PAR ^ 1, I3{});
-    phase_schedule(I12{}, I1{}, I1{}, I0{});
+    phase_schedule(VB{}, DR{}, I1{}, I0{});
     __builtin_amdgcn_sched_barrier(0);
 
     // every LDS write of tile kt + 1 is out and every read of tile kt has returned
@@ -277,7 +286,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
     // phase 4: last k-step from registers, first fragments of tile kt + 1
     mfma_step(1);
     load_frags(PAR ^ 1, 0, 0);
-    phase_schedule(I0{}, I1{}, I0{}, I0{});
+    phase_schedule(I0{}, DR{}, I0{}, I0{});
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -301,14 +310,14 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   }
   if (kt < ke) body(kt, I0{});
 
-  // ---- split-K tiles: fp32 partial to the workspace, last arriver finishes the tile ------
+  // ---- split-K tiles: fp32 partial to the workspace ------------------------------------
   if (part >= 0) {
     const int tl = nid - p.dp_tiles;
     float* tile_base = p.sk_part + (size_t)tl * p.sk_split * PF_SK_SLOT_FLOATS;
     float* mine = tile_base + (size_t)part * PF_SK_SLOT_FLOATS;
     // layout [group of four accumulator registers][thread]: coalesced 16-byte accesses
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -317,53 +326,14 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
           const f4 v = {acc[i][j][r], acc[i][j][r + 1], acc[i][j][r + 2], acc[i][j][r + 3]};
           *reinterpret_cast<f4*>(mine + ((size_t)q * 256 + tid) * 4) = v;
         }
-    // These workgroups live for hundreds of microseconds, so one release / acquire fence
-    // pair per workgroup (an L2 write-back, then an invalidate in the finisher) is cheap
-    // here, and the partial tiles can use ordinary cached 16-byte accesses.
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) s_last = (atomicAdd(p.sk_cnt + tl, 1) == p.sk_split - 1);
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    // sum in part order, own part included from memory: the result does not depend on who
-    // arrived last.  Group q of thread tid: tile (i, j) = q / 4, registers 4 (q % 4) ...
-    const int col_l = lane & 31, row_l = 4 * (lane >> 5);
-    const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
-    for (int q0 = 0; q0 < 64; q0 += 8) {   // eight groups x sk_split loads in flight
-      f4 v[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = f4{0.f, 0.f, 0.f, 0.f};
-      for (int s = 0; s < p.sk_split; ++s) {
-        f4 t[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-          t[u] = *reinterpret_cast<const f4*>(tile_base + (size_t)s * PF_SK_SLOT_FLOATS +
-                                              ((size_t)(q0 + u) * 256 + tid) * 4);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] += t[u];
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int q = q0 + u;
-        const int ij = q >> 2, r = (q & 3) * 4;
-        const int col = n0 + wn + 32 * (ij & 3) + col_l;
-        const int row = m0 + wm + 32 * (ij >> 2) + 8 * (r >> 2) + row_l;
-        if (col < p.N) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (row + e < p.M) p.y[(size_t)(row + e) * p.N + col] = (half_t)v[u][e];
-        }
-      }
-    }
-    if (tid == 0) p.sk_cnt[tl] = 0;
+    // summed and written out by awq_gemm_mfma_reduce_kernel, launched behind this kernel
     return;
   }
 
   // D[i][j] of a 32x32 tile: j = lane % 32, i = 8 * (r / 4) + 4 * (lane / 32) + r % 4
   const int col_l = lane & 31, row_l = 4 * (lane >> 5);
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int col = n0 + wn + 32 * j + col_l;
@@ -374,6 +344,52 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
         if (row < p.M) p.y[(size_t)row * p.N + col] = (half_t)acc[i][j][r];
       }
     }
+}
+
+// Sum of the split-K partial tiles.  Partial layout per (tile, part): [q][thread] groups of
+// four floats, q = (i * 4 + j) * 4 + r / 4 over the MI x 4 accumulator tiles of the producing
+// thread.  One workgroup takes four q of one tile; parts are added in index order.
+template <int MI>
+__global__ __launch_bounds__(256) void awq_gemm_mfma_reduce_kernel(const MfmaGemmParams p) {
+  constexpr int QPW = 4;
+  constexpr int QT = 16 * MI;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tl = blockIdx.x / (QT / QPW);
+  const int q0 = (blockIdx.x % (QT / QPW)) * QPW;
+  const int nid = p.dp_tiles + tl;
+  const int gsize = 8 * p.nt;
+  const int first_m = (nid / gsize) * 8;
+  const int gm = min(p.mt - first_m, 8);
+  const int mt_i = first_m + (nid % gsize) % gm;
+  const int nt_i = (nid % gsize) / gm;
+  const int m0 = mt_i * (64 * MI), n0 = nt_i * PF_BN;
+  const int wm = (wave >> 1) * (32 * MI), wn = (wave & 1) * 128;
+  const int col_l = lane & 31, row_l = 4 * (lane >> 5);
+  const float* tile_base = p.sk_part + (size_t)tl * p.sk_split * PF_SK_SLOT_FLOATS;
+  f4 v[QPW];
+#pragma unroll
+  for (int u = 0; u < QPW; ++u) v[u] = f4{0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < p.sk_split; ++s) {
+    f4 t[QPW];
+#pragma unroll
+    for (int u = 0; u < QPW; ++u)
+      t[u] = *reinterpret_cast<const f4*>(tile_base + (size_t)s * PF_SK_SLOT_FLOATS +
+                                          ((size_t)(q0 + u) * 256 + tid) * 4);
+#pragma unroll
+    for (int u = 0; u < QPW; ++u) v[u] += t[u];
+  }
+#pragma unroll
+  for (int u = 0; u < QPW; ++u) {
+    const int q = q0 + u;
+    const int ij = q >> 2, r = (q & 3) * 4;
+    const int col = n0 + wn + 32 * (ij & 3) + col_l;
+    const int row = m0 + wm + 32 * (ij >> 2) + 8 * (r >> 2) + row_l;
+    if (col < p.N) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (row + e < p.M) p.y[(size_t)(row + e) * p.N + col] = (half_t)v[u][e];
+    }
+  }
 }
 
 }  // namespace awqmi

@@ -179,6 +179,18 @@ def test_gemm_prefill(sba, gpu, M, K, N, G):
     _check_gemm(sba, gpu, x, qw, s, qz, K if G <= 0 else G, 0, tag="prefill")
 
 
+@pytest.mark.parametrize("M,K,N,G", [(65, 512, 512, 128), (100, 1024, 520, 128), (128, 2048, 1024, 128),
+                                     (96, 192, 264, 32), (127, 384, 256, -1), (128, 1024, 8192 + 256, 128)])
+def test_gemm_half_tile(sba, gpu, M, K, N, G):
+    """65 .. 128 rows run the 128-row workgroup tile (ragged rows / columns, K split included);
+    two runs agree bit for bit."""
+    x, qw, s, qz = _np_case(M, K, N, G, seed=M + K + 1)
+    g = K if G <= 0 else G
+    y1 = _check_gemm(sba, gpu, x, qw, s, qz, g, 0, tag="half-tile")
+    y2 = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), 0).cpu().numpy()
+    assert np.array_equal(y1.view(np.uint16), y2.view(np.uint16))
+
+
 @pytest.mark.parametrize("M,K,N", [(512, 1024, 1280), (300, 2048, 520), (2048, 512, 5120), (768, 1536, 8192 + 256)])
 def test_gemm_prefill_partial_rounds(sba, gpu, M, K, N):
     """Tile counts that are not a multiple of the CU count, ragged last row / column tiles;
