@@ -469,11 +469,11 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
       // per workgroup, which costs far more than the few KB of partials.
       float* mine = p.part + (((size_t)sp * ntiles + tile) * MB + mb) * TILE_F;
       const int nelem = rows * (NT * 16);
-      for (int i = tid * 4; i < nelem; i += 1024) {
+      // neighbouring lanes write neighbouring 8-byte pairs: whole 32-byte sectors per store
+      for (int i = tid * 2; i < nelem; i += 512) {
         const int m = i / (NT * 16), c = i % (NT * 16);
-        const f4 v = *reinterpret_cast<const f4*>(&red[0][m][c]) + *reinterpret_cast<const f4*>(&red[1][m][c]);
-        st_coherent(mine + i, f2{v[0], v[1]});
-        st_coherent(mine + i + 2, f2{v[2], v[3]});
+        const f2 v = *reinterpret_cast<const f2*>(&red[0][m][c]) + *reinterpret_cast<const f2*>(&red[1][m][c]);
+        st_coherent(mine + i, v);
       }
     } else {
       emit(mb, rows, true);
