@@ -254,8 +254,10 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   if (K % PF_BK == 0 && (pow2g || G % 64 == 0) && small) {
     static std::atomic<bool> attr_set{false};
     if (!attr_set.load(std::memory_order_acquire)) {
-      const void* fns[4] = {reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4>),
+      const void* fns[6] = {reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4>),
                             reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 4>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 3>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 3>),
                             reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 2>),
                             reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 2>)};
       for (const void* fn : fns) {
@@ -269,9 +271,9 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     p.M = M; p.K = K; p.N = N; p.NW = NW; p.G = G;
     p.gshift = 0;
     if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
-    // at most 128 rows: one row of 128-row tiles (half the MFMA work of a padded 256-row tile)
-    const bool half_tile = M <= 128;
-    p.mt = half_tile ? 1 : (M + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
+    // at most 128 / 192 rows: one row of 128- / 192-row tiles instead of a padded 256-row tile
+    const int mi = M <= 128 ? 2 : (M <= 192 ? 3 : 4);
+    p.mt = mi < 4 ? 1 : (M + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
     p.total = p.mt * p.nt;
     MfmaPlan pl = plan_mfma(M, K, N);
     // the K split needs the caller's workspace (counters + partial tiles); without it every
@@ -284,20 +286,19 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     p.sk_part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
                           : nullptr;
     const dim3 grid(p.per_xcd * 8 + p.sk_tiles * p.sk_split);
-    if (half_tile && pow2g)
-      hipLaunchKernelGGL((awq_gemm_mfma_kernel<true, 2>), grid, dim3(256), PF_LDS_BYTES, st, p);
-    else if (half_tile)
-      hipLaunchKernelGGL((awq_gemm_mfma_kernel<false, 2>), grid, dim3(256), PF_LDS_BYTES, st, p);
-    else if (pow2g)
-      hipLaunchKernelGGL((awq_gemm_mfma_kernel<true, 4>), grid, dim3(256), PF_LDS_BYTES, st, p);
-    else
-      hipLaunchKernelGGL((awq_gemm_mfma_kernel<false, 4>), grid, dim3(256), PF_LDS_BYTES, st, p);
-    if (p.sk_tiles > 0) {
-      if (half_tile)
-        hipLaunchKernelGGL(awq_gemm_mfma_reduce_kernel<2>, dim3(p.sk_tiles * 8), dim3(256), 0, st, p);
-      else
-        hipLaunchKernelGGL(awq_gemm_mfma_reduce_kernel<4>, dim3(p.sk_tiles * 16), dim3(256), 0, st, p);
-    }
+#define AWQMI_MFMA(MIV)                                                                            \
+  do {                                                                                           \
+    if (pow2g)                                                                                   \
+      hipLaunchKernelGGL((awq_gemm_mfma_kernel<true, MIV>), grid, dim3(256), PF_LDS_BYTES, st, p);  \
+    else                                                                                         \
+      hipLaunchKernelGGL((awq_gemm_mfma_kernel<false, MIV>), grid, dim3(256), PF_LDS_BYTES, st, p); \
+    if (p.sk_tiles > 0)                                                                          \
+      hipLaunchKernelGGL(awq_gemm_mfma_reduce_kernel<MIV>, dim3(p.sk_tiles * 4 * MIV), dim3(256), 0, st, p); \
+  } while (0)
+    if (mi == 2) AWQMI_MFMA(2);
+    else if (mi == 3) AWQMI_MFMA(3);
+    else AWQMI_MFMA(4);
+#undef AWQMI_MFMA
     return launch_status();
   }
 

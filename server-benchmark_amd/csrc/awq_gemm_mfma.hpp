@@ -69,9 +69,9 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* base, size
 // POW2G: G is a power of two (group index by shift, any G >= 8); otherwise G % 64 == 0 and
 // a k-tile lies inside one group (group index on the scalar unit).
 //
-// MI = 32-row MFMA tiles per wave along M: 4 gives the 256-row workgroup tile; 2 gives a
-// 128-row tile (each wave 64 x 128) for launches of at most 128 rows, which would leave half
-// of a 256-row tile multiplying padding.
+// MI = 32-row MFMA tiles per wave along M: 4 gives the 256-row workgroup tile; 3 and 2 give
+// 192- and 128-row tiles (each wave 96 x 128 / 64 x 128) for launches of at most that many
+// rows, which would leave part of a 256-row tile multiplying padding.
 template <bool POW2G, int MI = 4>
 __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmParams p) {
   constexpr int BM = 64 * MI;      // workgroup tile rows
@@ -134,9 +134,15 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   // u = hh ^ swz(i) the physical slot is u ^ (2 ks) ^ (4 (tile & 1)): four lane offsets
   const int fi = lane & 31, fh = lane >> 5;
   const int fu = fh ^ pf_swz(fi);
-  int f_off[4];
+  int f_off[4], fa_off[4];
+  // a wave whose first X row is an odd multiple of 32 (192-row tile, second wave row) sees
+  // the swizzle of its rows flipped in bit 2
+  const int fua = fu ^ (((wm >> 5) & 1) << 2);
 #pragma unroll
-  for (int c = 0; c < 4; ++c) f_off[c] = fi * PF_ROW_BYTES + ((fu ^ (2 * c)) << 4);
+  for (int c = 0; c < 4; ++c) {
+    f_off[c] = fi * PF_ROW_BYTES + ((fu ^ (2 * c)) << 4);
+    fa_off[c] = fi * PF_ROW_BYTES + ((fua ^ (2 * c)) << 4);
+  }
 
   f16v acc[MI][4];
 #pragma unroll
@@ -206,7 +212,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
     const unsigned char* bs = Bs + buf * PF_TILE_BYTES + wn * PF_ROW_BYTES;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
-      af[fs][i] = *reinterpret_cast<const h8*>(as + 32 * i * PF_ROW_BYTES + f_off[ks ^ (2 * (i & 1))]);
+      af[fs][i] = *reinterpret_cast<const h8*>(as + 32 * i * PF_ROW_BYTES + fa_off[ks ^ (2 * (i & 1))]);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       bf[fs][j] = *reinterpret_cast<const h8*>(bs + 32 * j * PF_ROW_BYTES + f_off[ks ^ (2 * (j & 1))]);
@@ -242,11 +248,11 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
   // per-MFMA-pair shares; the 128-row tile has half the MFMAs per phase for the same W work
-  using VA = std::integral_constant<int, MI == 4 ? 6 : 12>;    // dequant VALU, phases 1 and 2
-  using VB = std::integral_constant<int, MI == 4 ? 12 : 24>;   // phase 3
-  using DR = std::integral_constant<int, MI == 4 ? 1 : 2>;     // fragment reads
-  using DW1 = std::integral_constant<int, MI == 4 ? 1 : 3>;    // LDS writes, phase 1 (X tile + byte 0)
-  using VM1 = std::integral_constant<int, MI == 4 ? 2 : 3>;    // W / zero / scale loads, phase 1
+  using VA = std::integral_constant<int, 48 / (2 * MI)>;             // dequant VALU, phases 1 and 2
+  using VB = std::integral_constant<int, 96 / (2 * MI)>;             // phase 3
+  using DR = std::integral_constant<int, MI == 4 ? 1 : 2>;           // fragment reads
+  using DW1 = std::integral_constant<int, MI == 4 ? 1 : (MI == 3 ? 2 : 3)>;  // LDS writes, phase 1 (X tile + byte 0)
+  using VM1 = std::integral_constant<int, MI == 2 ? 3 : 2>;          // W / zero / scale loads, phase 1
 
   // One k-tile, PAR = kt & 1.  On entry: LDS buffer PAR holds tile kt and fragment set 0 its
   // first k-step; areg and W set PAR^1 hold tile kt + 1; W set PAR is free.  Tiles past the

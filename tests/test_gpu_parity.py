@@ -180,9 +180,11 @@ def test_gemm_prefill(sba, gpu, M, K, N, G):
 
 
 @pytest.mark.parametrize("M,K,N,G", [(65, 512, 512, 128), (100, 1024, 520, 128), (128, 2048, 1024, 128),
-                                     (96, 192, 264, 32), (127, 384, 256, -1), (128, 1024, 8192 + 256, 128)])
+                                     (96, 192, 264, 32), (127, 384, 256, -1), (128, 1024, 8192 + 256, 128),
+                                     (129, 512, 512, 128), (160, 1024, 520, 64), (192, 2048, 1024, 128),
+                                     (190, 512, 8192 + 256, 128)])
 def test_gemm_half_tile(sba, gpu, M, K, N, G):
-    """65 .. 128 rows run the 128-row workgroup tile (ragged rows / columns, K split included);
+    """65 .. 192 rows run the 128- / 192-row workgroup tile (ragged rows / columns, K split included);
     two runs agree bit for bit."""
     x, qw, s, qz = _np_case(M, K, N, G, seed=M + K + 1)
     g = K if G <= 0 else G
