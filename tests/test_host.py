@@ -210,3 +210,25 @@ def test_workload_pack_matches_oracle(sba):
     from oracle import awq_ref
     v = torch.randint(0, 16, (5, 64), generator=torch.Generator().manual_seed(1))
     assert np.array_equal(sba.workloads.pack_int4_awq(v).numpy(), awq_ref.pack_awq(v.numpy()))
+
+
+def test_vllm_plugin_rebinds_ops(sba, monkeypatch):
+    """Against a stand-in `vllm._custom_ops`: both ops are rebound to this package's functions
+    (same argument order as vLLM's); without vLLM the plugin raises ImportError."""
+    import importlib, inspect, sys, types
+    plugin = importlib.import_module(sba.__name__ + ".vllm_plugin")
+    monkeypatch.delitem(sys.modules, "vllm", raising=False)
+    monkeypatch.delitem(sys.modules, "vllm._custom_ops", raising=False)
+    with pytest.raises(ImportError):
+        plugin.register()
+    vllm = types.ModuleType("vllm")
+    vllm.__path__ = []
+    ops_mod = types.ModuleType("vllm._custom_ops")
+    ops_mod.awq_gemm = ops_mod.awq_dequantize = lambda *a: (_ for _ in ()).throw(AssertionError("old op"))
+    monkeypatch.setitem(sys.modules, "vllm", vllm)
+    monkeypatch.setitem(sys.modules, "vllm._custom_ops", ops_mod)
+    assert plugin.register() == ["awq_dequantize", "awq_gemm"]
+    assert ops_mod.awq_gemm is sba.awq_gemm and ops_mod.awq_dequantize is sba.awq_dequantize
+    assert list(inspect.signature(ops_mod.awq_gemm).parameters)[:5] == \
+        ["input", "qweight", "scales", "qzeros", "split_k_iters"]
+    assert list(inspect.signature(ops_mod.awq_dequantize).parameters)[:3] == ["qweight", "scales", "zeros"]
