@@ -392,6 +392,7 @@ def main():
         out["decoder"] = res
         log(f"[bench] decoder: prefill {res['prefill_s']} s, {res['ms_per_decode_step']} ms/decode step, "
             f"{res['output_tokens_per_s']} output tok/s")
+        log(import_module(sba.__name__ + ".report").format_serving_result(res))
 
     # ------------------------------------------------------------------ CPU baseline leg
     if not args.no_cpu:
