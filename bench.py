@@ -197,7 +197,7 @@ def main():
     # per-point detail (direct launches, event pair per point, same rotation)
     points = []
     stream_ptr = torch.cuda.current_stream().cuda_stream
-    reps = 10
+    reps = 50          # per point: 50 timed launches (the sweep before this was the warm-up), median + p10 / p90
     for name, K, N in ([] if args.sweep_only else layers):
         for ci, M in enumerate(Ms):
             # flush the last-level cache with the other layers' copies between points
@@ -216,6 +216,7 @@ def main():
             med = ts[len(ts) // 2]
             nbytes = workloads.linear_bytes(M, K, N, G)
             points.append({"layer": name, "M": M, "K": K, "N": N, "us": round(med, 2),
+                           "us_p10": round(ts[len(ts) // 10], 2), "us_p90": round(ts[(9 * len(ts)) // 10], 2),
                            "GBps": round(nbytes / med / 1e3, 1),
                            "frac_hbm": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4),
                            "split_k": lib.awqmi_gemm_auto_split_k(M, K, N, G) if args.split_k == 0 else args.split_k})
@@ -233,13 +234,19 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int4 weights x fp16 activations, fp32 accumulate",
+        "dtype": "f16 (int4 weights dequantised to f16, f32 accumulate)",
         "data": "synthetic: on-device seeded uniform int4 weights/zeros in AWQ packing, "
                 "U[0.001,0.02] fp16 scales, N(0,1) fp16 activations",
         "config": {"workload": "decode GEMV sweep, Qwen2.5-72B AWQ layer shapes (qkv 8192x10240, o 8192x8192, "
                                "gate_up 8192x59136, down 29568x8192), group 128, M in {1,4,8,16}; "
                                "16 awq_gemm launches per step, 4 rotating weight copies per layer",
                    "launch": args.launch, "split_k": args.split_k, "bytes_per_step": step_bytes},
+        "peaks": {"hbm_GBps": HBM_PEAK_GBS, "hbm_source": "MI355X published HBM3E bandwidth, 8 TB/s",
+                  "mfma_fp16_TFLOPs": MFMA_FP16_PEAK_TFLOPS,
+                  "mfma_source": "256 CUs x 4096 fp16 flop/clk/CU (dense MFMA) x 2.4 GHz = 2516.6 TFLOP/s, "
+                                 "quoted as 2.5 PFLOP/s",
+                  "device": torch.cuda.get_device_name(dev),
+                  "compute_units": torch.cuda.get_device_properties(dev).multi_processor_count},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": DECODE_SWEEP_TRAFFIC_BYTES if args.split_k == 0 and args.variant < 0 else None,
@@ -370,7 +377,7 @@ def main():
             fl = workloads.moe_flops(T, topk, H, I)
             mo.append({"T": T, "distinct_experts": distinct, "us": round(us, 1), "us_eager_call": round(us_eager, 1),
                        "GBps": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-                       "TFLOPs": round(fl / us / 1e6, 2)})
+                       "TFLOPs": round(fl / us / 1e6, 2), "frac_mfma": round(fl / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 5)})
             if args.detail:
                 log(f"   moe T={T:4d} experts hit {distinct:3d}  {us:9.1f} us (eager call {us_eager:6.1f})  "
                     f"{nbytes / us / 1e3:8.1f} GB/s")
@@ -418,6 +425,34 @@ def main():
             err = float((yg - yc.float()).norm() / yc.float().norm())
             worst = max(worst, err)
             del qw, sc, qz, yc
+        # the CPU-runnable configuration (M=16, K=N=4096, seed 0, drawn on the CPU generator)
+        c0 = workloads.config0()
+        g0 = c0.to(dev)
+        for _ in range(10):
+            y0 = sba.awq_gemm(g0.x, g0.qweight, g0.scales, g0.qzeros, 0)
+        torch.cuda.synchronize()
+        evs = []
+        for _ in range(50):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            y0 = sba.awq_gemm(g0.x, g0.qweight, g0.scales, g0.qzeros, 0)
+            b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        t0s = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)
+        cpu_ts = []
+        for _ in range(7):
+            t1 = time.perf_counter()
+            yc0 = awq_ref.cpu_linear_torch(c0.x, c0.qweight, c0.scales, c0.qzeros, 128)
+            cpu_ts.append(time.perf_counter() - t1)
+        cpu_ts = sorted(cpu_ts[2:])
+        err0 = float((y0.float().cpu() - yc0.float()).norm() / yc0.float().norm())
+        out["config0"] = {"workload": "M=16, K=N=4096, group 128, seed 0 (cache-warm: 8.9 MB of weights)",
+                          "gpu_us_median": round(t0s[len(t0s) // 2], 2), "gpu_us_p10": round(t0s[5], 2),
+                          "gpu_us_p90": round(t0s[45], 2),
+                          "cpu_ms_median": round(cpu_ts[len(cpu_ts) // 2] * 1e3, 2), "cpu_threads": nthreads,
+                          "gpu_vs_cpu_rel_frobenius": round(err0, 6)}
+        worst = max(worst, err0)
         cpu_model = ""
         try:
             with open("/proc/cpuinfo") as f:
