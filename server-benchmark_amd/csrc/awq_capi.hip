@@ -81,12 +81,12 @@ inline size_t gemv_partial_bytes(int N, int split, long long blocks_z, int tile_
   return (size_t)split * (size_t)blocks_z * tile_m * npad * sizeof(float);
 }
 
-template <int WPL, int MB, bool MOE, int RING = 4>
+template <int WPL, int MB, bool MOE, int RING = 4, int KW = 4>
 void launch_gemv(const GemvParams& p, dim3 grid, hipStream_t st) {
-  if (p.G == 32) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MB, MOE, RING>), grid, dim3(256), 0, st, p);
-  else if (p.G == 64) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MB, MOE, RING>), grid, dim3(256), 0, st, p);
-  else if (p.G == 128) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MB, MOE, RING>), grid, dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MB, MOE, RING>), grid, dim3(256), 0, st, p);
+  if (p.G == 32) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MB, MOE, RING, KW>), grid, dim3(256), 0, st, p);
+  else if (p.G == 64) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MB, MOE, RING, KW>), grid, dim3(256), 0, st, p);
+  else if (p.G == 128) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MB, MOE, RING, KW>), grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MB, MOE, RING, KW>), grid, dim3(256), 0, st, p);
 }
 
 // rows the skinny kernel takes in one awq_gemm call (passes of up to 32 rows)
@@ -440,12 +440,18 @@ int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales
   // group blocks by XCD once experts average two blocks or more
   p.grp = (long long)n_slots >= 2LL * tile_m * E ? 8 : 1;
   if (variant >= 0 && ((variant >> 2) & 7)) p.grp = 1 << (((variant >> 2) & 7) - 1);
+  // few chunks of K and no split across workgroups: two column blocks per workgroup, two
+  // waves each (three chunks per wave at K = 768 instead of 2 / 2 / 1 / 1)
+  const bool pair_cols = tile_m == 16 && wpl == 2 && split == 1 && K / 128 <= 8 && (K / 128) % 2 == 0 &&
+                         !(variant >= 0 && (variant & 64));
+  const int ncg = pair_cols ? (ncb + 1) / 2 : ncb;
   // runs of grp slots, dealt to the 8 XCDs in turn; the last deal may be partial
-  const long long runs = (long long)(nblk / p.grp) * ncb * split;
+  const long long runs = (long long)(nblk / p.grp) * ncg * split;
   const dim3 grid((unsigned)((runs + 7) / 8 * 8 * p.grp));
   hipStream_t st = (hipStream_t)stream;
   if (tile_m == 32) launch_gemv<2, 2, true>(p, grid, st);
   else if (wpl == 2 && variant >= 0 && (variant & 2)) launch_gemv<2, 1, true, 4>(p, grid, st);
+  else if (pair_cols) launch_gemv<2, 1, true, 2, 2>(p, grid, st);
   else if (wpl == 2) launch_gemv<2, 1, true, 2>(p, grid, st);
   else launch_gemv<1, 1, true>(p, grid, st);
   return launch_status();

@@ -311,8 +311,13 @@ struct GemvWave {
   }
 };
 
-template <int WPL, int GMODE, int MB, bool MOE, int RING = 4>
+// KW = waves of a workgroup that share one column block and split its K range (4, or 2: the
+// workgroup then covers two neighbouring column blocks with two waves each, which keeps the
+// waves' ranges long and even when K is only a few chunks; launches with KW = 2 do not split K
+// across workgroups).
+template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4>
 __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
+  constexpr int CW = 4 / KW;       // column blocks per workgroup
   constexpr int NT = 8 * WPL;
   constexpr int CB = 128 * WPL;
   constexpr int RS = NT * 16 + 4;  // LDS row stride in floats: 4h rows land 16 banks apart
@@ -333,10 +338,10 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
     const int B = p.grp;
     const int lin = blockIdx.x, xcd = lin & 7, slot = lin >> 3;
     const int g = (slot / B) * 8 + xcd;            // run index: (block group, column block, part)
-    const int ncbs = p.ncb * p.split_k;
+    const int ncbs = ((p.ncb + CW - 1) / CW) * p.split_k;
     const int bg = g / ncbs, cbs = g % ncbs;
     blk = bg * B + slot % B;
-    cb = cbs / p.split_k;
+    cb = cbs / p.split_k;          // column group of the workgroup (a column block when CW = 1)
     sp = cbs % p.split_k;
     if (blk >= p.nblk || blk * TM >= *p.n_post_pad) return;
     const int e = p.expert_ids[blk];
@@ -360,7 +365,9 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
 
   // Lanes past the last word column / past the last row read valid memory of column block 0
   // / row 0 instead; their B column (resp. A row) only feeds outputs that are never stored.
-  int wc = cb * (16 * WPL) + WPL * j;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int cbw = cb * CW + wave_u / KW;     // this wave's column block
+  int wc = cbw * (16 * WPL) + WPL * j;
   if (wc >= p.NW) wc = 0;
 
   GemvWave<WPL, GMODE, MB, RING> w;
@@ -387,9 +394,8 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
 
   // this wave's share of K, in 128-row chunks; the wave index is made scalar so that the
   // row base addresses stay in SGPRs
-  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-  const long long parts = 4LL * p.split_k;
-  const long long pw = (long long)sp * 4 + wave_u;
+  const long long parts = (long long)KW * p.split_k;
+  const long long pw = (long long)sp * KW + wave_u % KW;
   const int nchunks = p.K / 128;
   const int c_begin = (int)(pw * nchunks / parts);
   const int c_end = (int)((pw + 1) * nchunks / parts);
@@ -406,18 +412,19 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
 
   // tile-major LDS (red[0], optionally + red[1]) -> row-major fp16 output of row block mb;
   // one thread gathers the eight columns of a packed word and stores them as 16 bytes
-  auto emit = [&](int mb, int rows, bool two) {
+  auto emit = [&](int mb, int rows, bool two, int buf = 0, int cbo = -1) {
     constexpr int WPB = 16 * WPL;   // packed words per row of the block
+    if (cbo < 0) cbo = cb;
     for (int it = tid; it < rows * WPB; it += 256) {
       const int m = it / WPB, wl = it % WPB;
       const int jj = wl / WPL, ww = wl % WPL;
-      const int col = cb * CB + wl * 8;
+      const int col = cbo * CB + wl * 8;
       if (col >= p.N) continue;
       float v[8];
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         const int t = ww * 8 + awq_nibble_of_col(c);
-        v[c] = red[0][m][t * 16 + jj];
+        v[c] = red[buf][m][t * 16 + jj];
         if (two) v[c] += red[1][m][t * 16 + jj];
       }
       size_t orow = (size_t)(mb * 16 + m);
@@ -439,6 +446,32 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int rows = min(16, max(0, rows_total - 16 * mb));
+    if (KW == 2) {
+      // two column blocks, two waves each: the odd wave of a pair writes, the even one adds,
+      // and each buffer is written out on its own
+      if (wave & 1) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (4 * h + r < rows) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) red[wave >> 1][4 * h + r][t * 16 + j] = w.acc[mb][t][r];
+          }
+      }
+      __syncthreads();
+      if (!(wave & 1)) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (4 * h + r < rows) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) red[wave >> 1][4 * h + r][t * 16 + j] += w.acc[mb][t][r];
+          }
+      }
+      __syncthreads();
+      emit(mb, rows, false, 0, cb * 2);
+      if (cb * 2 + 1 < p.ncb) emit(mb, rows, false, 1, cb * 2 + 1);
+      __syncthreads();
+      continue;
+    }
     // ---- cross-wave sum in LDS: red[b][row][tile*16 + j] ----
     // (rows past the block's last one are never read back)
     if (wave >= 2) {
