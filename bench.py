@@ -74,8 +74,9 @@ def main():
     args = ap.parse_args()
 
     if args.gpus != 1:
-        log("bench.py: this build measures one GPU only (the path shards without changing the "
-            "kernel; see DESIGN.md).  Run with --gpus 1.")
+        log("bench.py: this build measures one GPU only: column-parallel layers shard the weight "
+            "triple on N with no exchange, row-parallel layers shard K and add one all-reduce, "
+            "and the kernels take a shard's shape as it is.  Run with --gpus 1.")
         sys.exit(2)
 
     import torch

@@ -160,7 +160,7 @@ def moe_forward(x, w13, w2, topk_ids, topk_w, group: int) -> np.ndarray:
 # --------------------------------------------------------------------------- baseline
 
 def cpu_linear_torch(x_t, qweight_t, scales_t, qzeros_t, group: int):
-    """The reference CPU path as BASELINE.json configs[0] states it: PyTorch dequantize
+    """The reference CPU path (M=16, K=N=4096 is its CPU-runnable case): PyTorch dequantize
     then matmul on the host.  Takes and returns torch CPU tensors."""
     import torch
 
