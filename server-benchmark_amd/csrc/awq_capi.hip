@@ -102,6 +102,14 @@ inline bool skinny_rows(int M, int N) {
 // Work split of the MFMA kernel: whole rounds of 256 tiles run one workgroup per tile; a
 // last round of fewer than 129 tiles (and any launch that small) is split in K over
 // floor(256 / tiles) workgroups per tile (at most 8, at least 8 k-tiles each).
+// The MFMA kernel addresses X through 32-bit buffer offsets: calls with more than 4 GiB of
+// activations run as consecutive row slabs (multiples of 256 rows).
+inline int mfma_slab_rows(int M, int K) {
+  const long long fit = ((1LL << 32) - 1) / ((long long)K * 2);
+  const long long rows = fit / 256 * 256;
+  return rows <= 0 ? 0 : (int)(rows < M ? rows : M);
+}
+
 struct MfmaPlan { int dp_tiles, sk_tiles, sk_split; size_t part_bytes; };
 MfmaPlan plan_mfma(int M, int K, int N) {
   const int mt = (M + PF_BM - 1) / PF_BM, nt = (N + PF_BN - 1) / PF_BN;
@@ -181,7 +189,16 @@ size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
   if (M <= 0 || K <= 0 || N <= 0) return 0;
   // the group size decides between the kernels for some shapes, so cover both
   size_t mfma = 0, skinny = 0;
-  if (M > 16 && K % PF_BK == 0) mfma = plan_mfma(M, K, N).part_bytes;
+  if (M > 16 && K % PF_BK == 0) {
+    const int slab = mfma_slab_rows(M, K);
+    if (slab > 0) {
+      mfma = plan_mfma(slab, K, N).part_bytes;
+      if (M % slab) {
+        const size_t last = plan_mfma(M % slab, K, N).part_bytes;
+        if (last > mfma) mfma = last;
+      }
+    }
+  }
   if (M <= SKINNY_MAX_M) {
     int s = split_k;
     if (s <= 0) s = (K % 128 == 0) ? pick_split_k(M, K, N, 128, 1) : 1;
@@ -211,7 +228,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
 
   const int wpl = gemv_wpl(N);
   const bool mfma_ok = K % PF_BK == 0 && (((G & (G - 1)) == 0 && G >= 8) || G % 64 == 0) &&
-                       (size_t)M * K * 2 < (1ull << 32) && (size_t)K * NW * 4 < (1ull << 32) &&
+                       mfma_slab_rows(M, K) > 0 && (size_t)K * NW * 4 < (1ull << 32) &&
                        (size_t)(K / G) * N * 2 < (1ull << 32);
   if (gemv_tiled_ok(K, G) &&
       (M <= 16 || (M <= SKINNY_MAX_M && wpl == 2 && (skinny_rows(M, N) || !mfma_ok)))) {
@@ -249,9 +266,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   // MFMA kernel: K % 64 == 0, G a power of two >= 8 or a multiple of 64; buffer offsets are
   // 32-bit, so every operand must stay below 4 GiB
   const bool pow2g = (G & (G - 1)) == 0 && G >= 8;
-  const bool small = (size_t)M * K * 2 < (1ull << 32) && (size_t)K * NW * 4 < (1ull << 32) &&
-                     (size_t)(K / G) * N * 2 < (1ull << 32);
-  if (K % PF_BK == 0 && (pow2g || G % 64 == 0) && small) {
+  if (mfma_ok) {
     static std::atomic<bool> attr_set{false};
     if (!attr_set.load(std::memory_order_acquire)) {
       const void* fns[6] = {reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4>),
@@ -266,16 +281,19 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
       }
       attr_set.store(true, std::memory_order_release);
     }
+    const int slab = mfma_slab_rows(M, K);
+    for (int r0 = 0; r0 < M; r0 += slab) {
+    const int Ms = M - r0 < slab ? M - r0 : slab;
     MfmaGemmParams p{};
-    p.x = xx; p.qw = qw; p.sc = sc; p.qz = qz; p.y = yy;
-    p.M = M; p.K = K; p.N = N; p.NW = NW; p.G = G;
+    p.x = xx + (size_t)r0 * K; p.qw = qw; p.sc = sc; p.qz = qz; p.y = yy + (size_t)r0 * N;
+    p.M = Ms; p.K = K; p.N = N; p.NW = NW; p.G = G;
     p.gshift = 0;
     if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
     // at most 128 / 192 rows: one row of 128- / 192-row tiles instead of a padded 256-row tile
-    const int mi = M <= 128 ? 2 : (M <= 192 ? 3 : 4);
-    p.mt = mi < 4 ? 1 : (M + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
+    const int mi = Ms <= 128 ? 2 : (Ms <= 192 ? 3 : 4);
+    p.mt = mi < 4 ? 1 : (Ms + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
     p.total = p.mt * p.nt;
-    MfmaPlan pl = plan_mfma(M, K, N);
+    MfmaPlan pl = plan_mfma(Ms, K, N);
     // the K split needs the caller's workspace (counters + partial tiles); without it every
     // tile runs on one workgroup
     if (pl.sk_tiles > 0 && (!workspace || !aligned16(workspace) ||
@@ -299,6 +317,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     else if (mi == 3) AWQMI_MFMA(3);
     else AWQMI_MFMA(4);
 #undef AWQMI_MFMA
+    }
     return launch_status();
   }
 

@@ -66,3 +66,19 @@ def test_prefill_sizes_against_dequant_matmul(sba, gpu, name, K, N, M):
     assert worst <= TOL
     y2 = sba.awq_gemm(x, qw, sc, qz, 0)
     assert torch.equal(y, y2)          # deterministic
+
+
+def test_activations_beyond_4gib_run_as_row_slabs(sba, gpu):
+    """X larger than the 32-bit buffer range of the MFMA kernel: the call is cut into row slabs;
+    checked on the rows around the cut and at both ends."""
+    K, N = 29568, 256
+    M = 72448 + 300                      # 72448 = largest multiple of 256 rows below 4 GiB / (2 K)
+    qw, sc, qz, g = _weights(K, N, gpu, 3)
+    W = sba.awq_dequantize(qw, sc, qz).float()
+    x = torch.randn((M, K), device=gpu, generator=g, dtype=torch.float16)
+    y = sba.awq_gemm(x, qw, sc, qz, 0)
+    for r0 in (0, 72448 - 256, 72448, M - 256):
+        ref = x[r0:r0 + 256].float() @ W
+        err = _rel(y[r0:r0 + 256], ref)
+        print(f"[slabs] rows {r0}..{r0 + 255} rel_fro={err:.2e}", flush=True)
+        assert err <= TOL
