@@ -71,10 +71,10 @@ size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k);
  * Stands in for vLLM's `awq_gemm` op (every AWQ Linear at decode and prefill); reached
  * from the server started at reference utils/generate_compose.py:85-93.
  * fp32 accumulation, one final rounding to fp16.  M >= 1; K % group == 0; N % 8 == 0.
- * M <= 32 takes the HBM-bound skinny kernel (split_k honoured, 0 = auto); 33 .. 64 rows take
+ * M <= 32 takes the HBM-bound skinny kernel (split_k honoured, 0 = auto); 33 .. 48 rows take
  * two skinny passes on very wide layers and the MFMA kernel otherwise; larger M the
- * LDS-dequant MFMA kernel (split_k ignored; 128- / 192-row tiles up to M = 128 / 192, 256-row
- * tiles above;
+ * LDS-dequant MFMA kernel (split_k ignored; 64- / 128- / 192-row tiles up to M = 64 / 128 /
+ * 192, 256-row tiles above;
  * when the workspace is at least awqmi_gemm_workspace_bytes() a sparsely filled last round
  * of tiles is split in K and a second short kernel sums the partial tiles, otherwise every
  * tile runs on one workgroup).  Shapes outside the fast kernels' tiling (K % 128 != 0, group

@@ -92,11 +92,11 @@ void launch_gemv(const GemvParams& p, dim3 grid, hipStream_t st) {
 // rows the skinny kernel takes in one awq_gemm call (passes of up to 32 rows)
 constexpr int SKINNY_MAX_M = 64;
 
-// Between 33 and 64 rows two skinny passes compete with the 128-row MFMA tile: the MFMA
-// kernel wins while its tiles (times the K split) fit one round of workgroups, the skinny
-// kernel wins on very wide layers, where the MFMA tiles alone fill the chip.
+// Between 33 and 64 rows two skinny passes compete with the 64-row MFMA tile: the MFMA
+// kernel wins while its tiles (times the K split) fit one round of workgroups; on very wide
+// layers, where the MFMA tiles alone fill the chip, the skinny kernel still wins up to 48 rows.
 inline bool skinny_rows(int M, int N) {
-  return M <= 32 || (M <= SKINNY_MAX_M && (N + 255) / 256 > 128);
+  return M <= 32 || (M <= 48 && (N + 255) / 256 > 128);
 }
 
 // Work split of the MFMA kernel: whole rounds of 256 tiles run one workgroup per tile; a
@@ -269,7 +269,9 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   if (mfma_ok) {
     static std::atomic<bool> attr_set{false};
     if (!attr_set.load(std::memory_order_acquire)) {
-      const void* fns[6] = {reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4>),
+      const void* fns[8] = {reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4>),
                             reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 4>),
                             reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 3>),
                             reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 3>),
@@ -289,8 +291,8 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     p.M = Ms; p.K = K; p.N = N; p.NW = NW; p.G = G;
     p.gshift = 0;
     if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
-    // at most 128 / 192 rows: one row of 128- / 192-row tiles instead of a padded 256-row tile
-    const int mi = Ms <= 128 ? 2 : (Ms <= 192 ? 3 : 4);
+    // at most 64 / 128 / 192 rows: one row of smaller tiles instead of a padded 256-row tile
+    const int mi = Ms <= 64 ? 1 : (Ms <= 128 ? 2 : (Ms <= 192 ? 3 : 4));
     p.mt = mi < 4 ? 1 : (Ms + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
     p.total = p.mt * p.nt;
     MfmaPlan pl = plan_mfma(Ms, K, N);
@@ -313,7 +315,8 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     if (p.sk_tiles > 0)                                                                          \
       hipLaunchKernelGGL(awq_gemm_mfma_reduce_kernel<MIV>, dim3(p.sk_tiles * 4 * MIV), dim3(256), 0, st, p); \
   } while (0)
-    if (mi == 2) AWQMI_MFMA(2);
+    if (mi == 1) AWQMI_MFMA(1);
+    else if (mi == 2) AWQMI_MFMA(2);
     else if (mi == 3) AWQMI_MFMA(3);
     else AWQMI_MFMA(4);
 #undef AWQMI_MFMA

@@ -69,8 +69,8 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* base, size
 // POW2G: G is a power of two (group index by shift, any G >= 8); otherwise G % 64 == 0 and
 // a k-tile lies inside one group (group index on the scalar unit).
 //
-// MI = 32-row MFMA tiles per wave along M: 4 gives the 256-row workgroup tile; 3 and 2 give
-// 192- and 128-row tiles (each wave 96 x 128 / 64 x 128) for launches of at most that many
+// MI = 32-row MFMA tiles per wave along M: 4 gives the 256-row workgroup tile; 3, 2 and 1
+// give 192-, 128- and 64-row tiles (each wave 32 MI x 128) for launches of at most that many
 // rows, which would leave part of a 256-row tile multiplying padding.
 template <bool POW2G, int MI = 4>
 __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmParams p) {
@@ -250,9 +250,9 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   // per-MFMA-pair shares; the 128-row tile has half the MFMAs per phase for the same W work
   using VA = std::integral_constant<int, 48 / (2 * MI)>;             // dequant VALU, phases 1 and 2
   using VB = std::integral_constant<int, 96 / (2 * MI)>;             // phase 3
-  using DR = std::integral_constant<int, MI == 4 ? 1 : 2>;           // fragment reads
-  using DW1 = std::integral_constant<int, MI == 4 ? 1 : (MI == 3 ? 2 : 3)>;  // LDS writes, phase 1 (X tile + byte 0)
-  using VM1 = std::integral_constant<int, MI == 2 ? 3 : 2>;          // W / zero / scale loads, phase 1
+  using DR = std::integral_constant<int, MI == 4 ? 1 : (MI == 1 ? 3 : 2)>;   // fragment reads
+  using DW1 = std::integral_constant<int, MI == 4 ? 1 : (MI == 3 ? 2 : (MI == 2 ? 3 : 4))>;  // LDS writes, phase 1 (X tile + byte 0)
+  using VM1 = std::integral_constant<int, MI == 2 ? 3 : (MI == 1 ? 6 : 2)>;   // W / zero / scale loads, phase 1
 
   // One k-tile, PAR = kt & 1.  On entry: LDS buffer PAR holds tile kt and fragment set 0 its
   // first k-step; areg and W set PAR^1 hold tile kt + 1; W set PAR is free.  Tiles past the
