@@ -1,0 +1,66 @@
+"""ROCm deployment description against a compose file the harness recorded
+(tests/golden/compose/*.yml is the "Docker Compose Configuration" block of one of its result
+files, 4 instances x 1 GPU behind nginx): everything that does not depend on the GPU vendor
+must come out the same; the GPU plumbing must be ROCm's."""
+import pathlib
+from importlib import import_module
+
+import pytest
+import yaml
+
+GOLD = pathlib.Path(__file__).parent / "golden" / "compose" / "rtx5090_x_4_qwen3_coder_30b_awq.yml"
+MODEL = "QuantTrio/Qwen3-Coder-30B-A3B-Instruct-AWQ"
+
+
+@pytest.fixture(scope="module")
+def deploy(sba):
+    return import_module(sba.__name__ + ".deploy")
+
+
+@pytest.fixture(scope="module")
+def stack(deploy):
+    return deploy.compose(4, 1, 1, "vllm_benchmark_container", f"/hf_models/{MODEL}", MODEL, "/hf_models",
+                          nginx_conf_path="/home/riftuser/server-benchmark/nginx.vllm.conf",
+                          extra_args="--max-model-len 8192", total_gpus=4)
+
+
+def test_vendor_independent_parts_match_the_recorded_stack(deploy, stack):
+    want = yaml.safe_load(GOLD.read_text())["services"]
+    got = yaml.safe_load(deploy.to_yaml(stack))["services"]          # through the YAML text
+    assert list(got) == list(want)
+    for i in range(4):
+        g, w = got[f"vllm_{i}"], want[f"vllm_{i}"]
+        for key in ("container_name", "ports", "shm_size", "ipc", "healthcheck"):
+            assert g[key] == w[key], key
+        assert g["command"].split() == w["command"].split()
+        assert g["volumes"][0] == w["volumes"][0]
+        assert g["environment"][0] == w["environment"][0]
+    assert got["nginx"] == want["nginx"]
+    for key in ("container_name", "volumes", "entrypoint", "command", "profiles"):
+        assert got["benchmark"][key] == want["benchmark"][key]
+
+
+def test_gpu_plumbing_is_rocm(deploy, stack):
+    for i in range(4):
+        s = stack["services"][f"vllm_{i}"]
+        assert s["devices"] == ["/dev/kfd:/dev/kfd", "/dev/dri:/dev/dri"] and s["group_add"] == ["video"]
+        assert f"HIP_VISIBLE_DEVICES={i}" in s["environment"]
+        assert "deploy" not in s and not any("CUDA" in e or "NVIDIA" in e for e in s["environment"])
+    one = deploy.compose(1, 8, 1, "c", "/m", "m", "/hf", total_gpus=8, library_dir="/srv/awq")
+    s = one["services"]["vllm_0"]
+    assert not any(e.startswith("HIP_VISIBLE_DEVICES") for e in s["environment"])      # sees every GPU
+    assert "/srv/awq:/opt/awq_mi355x:ro" in s["volumes"] and "VLLM_USE_TRITON_AWQ=0" in s["environment"]
+    assert "nginx" not in one["services"]
+    two = deploy.compose(2, 2, 2, "c", "/m", "m", "/hf", total_gpus=8)
+    assert "HIP_VISIBLE_DEVICES=4,5,6,7" in two["services"]["vllm_1"]["environment"]
+    with pytest.raises(ValueError):
+        deploy.compose(3, 4, 1, "c", "/m", "m", "/hf", total_gpus=8)
+
+
+def test_gpu_count_and_nginx_conf(deploy):
+    text = "\n".join(["Agent 1", "  Device Type:             CPU", "Agent 2", "  Device Type:             GPU",
+                      "  Compute Unit:            256", "Agent 3", "  Device Type:             GPU"])
+    assert deploy.count_rocm_gpus(text) == 2 and deploy.count_rocm_gpus("") == 0
+    conf = deploy.nginx_conf(3)
+    assert conf.count("server vllm_") == 3 and "least_conn;" in conf and "listen 8080;" in conf
+    assert "proxy_buffering off;" in conf and conf.count("{") == conf.count("}")
