@@ -269,7 +269,11 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   if (mfma_ok) {
     static std::atomic<bool> attr_set{false};
     if (!attr_set.load(std::memory_order_acquire)) {
-      const void* fns[8] = {reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1>),
+      const void* fns[12] = {reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1, 8>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1, 8>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 2, 8>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 2, 8>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1>),
                             reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1>),
                             reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4>),
                             reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 4>),
@@ -306,19 +310,24 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     p.sk_part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
                           : nullptr;
     const dim3 grid(p.per_xcd * 8 + p.sk_tiles * p.sk_split);
-#define AWQMI_MFMA(MIV)                                                                            \
+#define AWQMI_MFMA(MIV, NWVV)                                                                      \
   do {                                                                                           \
     if (pow2g)                                                                                   \
-      hipLaunchKernelGGL((awq_gemm_mfma_kernel<true, MIV>), grid, dim3(256), PF_LDS_BYTES, st, p);  \
+      hipLaunchKernelGGL((awq_gemm_mfma_kernel<true, MIV, NWVV>), grid, dim3(64 * NWVV), PF_LDS_BYTES, st, p);  \
     else                                                                                         \
-      hipLaunchKernelGGL((awq_gemm_mfma_kernel<false, MIV>), grid, dim3(256), PF_LDS_BYTES, st, p); \
+      hipLaunchKernelGGL((awq_gemm_mfma_kernel<false, MIV, NWVV>), grid, dim3(64 * NWVV), PF_LDS_BYTES, st, p); \
     if (p.sk_tiles > 0)                                                                          \
-      hipLaunchKernelGGL(awq_gemm_mfma_reduce_kernel<MIV>, dim3(p.sk_tiles * 4 * MIV), dim3(256), 0, st, p); \
+      hipLaunchKernelGGL((awq_gemm_mfma_reduce_kernel<MIV, NWVV>), dim3(p.sk_tiles * MIV * (16 / NWVV)),       \
+                         dim3(64 * NWVV), 0, st, p);                                              \
   } while (0)
-    if (mi == 1) AWQMI_MFMA(1);
-    else if (mi == 2) AWQMI_MFMA(2);
-    else if (mi == 3) AWQMI_MFMA(3);
-    else AWQMI_MFMA(4);
+    const bool eight = !(g_gemv_variant.load(std::memory_order_relaxed) >= 0 &&
+                         (g_gemv_variant.load(std::memory_order_relaxed) & 512));
+    if (mi == 1 && eight) AWQMI_MFMA(1, 8);
+    else if (mi == 2 && eight) AWQMI_MFMA(2, 8);
+    else if (mi == 1) AWQMI_MFMA(1, 4);
+    else if (mi == 2) AWQMI_MFMA(2, 4);
+    else if (mi == 3) AWQMI_MFMA(3, 4);
+    else AWQMI_MFMA(4, 4);
 #undef AWQMI_MFMA
     }
     return launch_status();

@@ -72,10 +72,20 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* base, size
 // MI = 32-row MFMA tiles per wave along M: 4 gives the 256-row workgroup tile; 3, 2 and 1
 // give 192-, 128- and 64-row tiles (each wave 32 MI x 128) for launches of at most that many
 // rows, which would leave part of a 256-row tile multiplying padding.
-template <bool POW2G, int MI = 4>
-__global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmParams p) {
-  constexpr int BM = 64 * MI;      // workgroup tile rows
-  constexpr int AL = 2 * MI;       // 16-byte X loads per thread and k-tile
+//
+// NWV = waves per workgroup.  4: one wave per SIMD, each 32 MI x 128 (the prefill
+// configuration: 256 accumulator registers per wave leave no room for a second wave).
+// 8: two waves per SIMD, each 32 MI x 64, for MI <= 2: with half the accumulators two waves
+// fit, and the waits of one (fragment reads, the barrier, operand loads) are covered by the
+// MFMAs of the other -- the small tiles spend most of a k-tile in such waits otherwise.
+template <bool POW2G, int MI = 4, int NWV = 4>
+__global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const MfmaGemmParams p) {
+  constexpr int BM = 64 * MI;            // workgroup tile rows
+  constexpr int NTH = 64 * NWV;          // threads
+  constexpr int NJ = 16 / NWV;           // 32-column MFMA tiles per wave (4 or 2)
+  constexpr int ARP = NTH / 8;           // X rows moved per pass of the workgroup
+  constexpr int AL = BM / ARP;           // 16-byte X loads per thread and k-tile
+  constexpr int RW = 2048 / NTH;         // rows of one word column a thread dequantises (8 or 4)
   extern __shared__ __align__(16) unsigned char smem_raw[];
   unsigned char* const As = smem_raw;                        // [2][256][128 B]
   unsigned char* const Bs = smem_raw + 2 * PF_TILE_BYTES;    // [2][256][128 B]
@@ -100,7 +110,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   const int mt_i = first_m + (nid % gsize) % gm;
   const int nt_i = (nid % gsize) / gm;
   const int m0 = mt_i * BM, n0 = nt_i * PF_BN;
-  const int wm = (wave >> 1) * (32 * MI), wn = (wave & 1) * 128;
+  const int wm = (wave / (NWV / 2)) * (32 * MI), wn = (wave % (NWV / 2)) * (32 * NJ);
 
   const __amdgpu_buffer_rsrc_t rx = pf_rsrc(p.x, (size_t)p.M * p.K * 2);
   const __amdgpu_buffer_rsrc_t rw = pf_rsrc(p.qw, (size_t)p.K * p.NW * 4);
@@ -115,18 +125,19 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   int a_dst[AL];
 #pragma unroll
   for (int i = 0; i < AL; ++i) {
-    const int r = a_row + 32 * i;
+    const int r = a_row + ARP * i;
     const int gr = min(m0 + r, p.M - 1);
     a_off[i] = (uint32_t)(((size_t)gr * p.K + 8 * a_seg) * 2);
     a_dst[i] = r * PF_ROW_BYTES + ((a_seg ^ pf_swz(r)) << 4);
   }
-  // W tile: thread (kk, wcl) takes rows 8kk..8kk+7 of word column wcl
+  // W tile: thread (kk, wcl) takes rows RW kk .. RW kk + RW - 1 of word column wcl
   const int kk = tid >> 5, wcl = tid & 31;
   int wcg = n0 / 8 + wcl;
   if (wcg >= p.NW) wcg = 0;                      // columns never stored; keep loads in bounds
-  const uint32_t w_off = (uint32_t)(((size_t)8 * kk * p.NW + wcg) * 4);
+  const uint32_t w_off = (uint32_t)(((size_t)RW * kk * p.NW + wcg) * 4);
   const uint32_t row_b = (uint32_t)p.NW * 4;     // bytes between qweight / qzeros rows
-  const int b_t = kk ^ (wcl & 7);                // physical slot of column c: b_t ^ c
+  const int b_t = (RW == 8 ? kk : (kk >> 1)) ^ (wcl & 7);   // physical 16-byte slot of column c: b_t ^ c
+  const int b_half = RW == 8 ? 0 : (kk & 1) * 8;            // 8-byte half of the slot (RW = 4)
   const int b_base = wcl * 8 * PF_ROW_BYTES;
 
   // ---- LDS -> fragment roles -----------------------------------------------------------
@@ -144,18 +155,18 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
     fa_off[c] = fi * PF_ROW_BYTES + ((fua ^ (2 * c)) << 4);
   }
 
-  f16v acc[MI][4];
+  f16v acc[MI][NJ];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   NibbleMasks nm;
   nm.init();
   u4v areg[AL];         // X tile in flight
-  uint32_t wreg[2][8];  // two W tiles in flight (parity of the k-tile)
+  uint32_t wreg[2][RW]; // two W tiles in flight (parity of the k-tile)
   uint32_t zreg[2];
   u4v sreg[2];
   auto gload_a = [&](int kt) {
@@ -166,10 +177,10 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   auto gload_w = [&](int kt, int set) {
     const uint32_t so = (uint32_t)kt * PF_BK * row_b;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < RW; ++i)
       wreg[set][i] = __builtin_amdgcn_raw_buffer_load_b32(rw, w_off, so + i * row_b, 0);
     if (POW2G) {
-      const uint32_t g = (uint32_t)(kt * PF_BK + 8 * kk) >> p.gshift;
+      const uint32_t g = (uint32_t)(kt * PF_BK + RW * kk) >> p.gshift;
       zreg[set] = __builtin_amdgcn_raw_buffer_load_b32(rz, g * row_b + wcg * 4, 0, 0);
       sreg[set] = __builtin_amdgcn_raw_buffer_load_b128(rs, (g * (uint32_t)p.N + 8 * wcg) * 2, 0, 0);
     } else {
@@ -195,18 +206,25 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
                                  : __builtin_amdgcn_perm(sw_l, sw_l, 0x01000100u);
     const uint32_t sh = (ch & 1) ? __builtin_amdgcn_perm(sw_h, sw_h, 0x03020302u)
                                  : __builtin_amdgcn_perm(sw_h, sw_h, 0x01000100u);
-    u4v lo, hi;
+    uint32_t lo[RW / 2], hi[RW / 2];
 #pragma unroll
-    for (int rp = 0; rp < 4; ++rp) {
+    for (int rp = 0; rp < RW / 2; ++rp) {
       const uint32_t t = byte_pair<B>(wreg[set][2 * rp + 1], wreg[set][2 * rp]);
       lo[rp] = pk_mul(pk_sub((t & nm.lo) | MAGIC_LO, zl), sl);
       hi[rp] = pk_mul(pk_sub((t & nm.hi) | MAGIC_HI, zh), sh);
     }
-    *reinterpret_cast<u4v*>(bs + b_base + cl * PF_ROW_BYTES + ((b_t ^ cl) << 4)) = lo;
-    *reinterpret_cast<u4v*>(bs + b_base + ch * PF_ROW_BYTES + ((b_t ^ ch) << 4)) = hi;
+    unsigned char* dl = bs + b_base + cl * PF_ROW_BYTES + ((b_t ^ cl) << 4) + b_half;
+    unsigned char* dh = bs + b_base + ch * PF_ROW_BYTES + ((b_t ^ ch) << 4) + b_half;
+    if constexpr (RW == 8) {
+      *reinterpret_cast<u4v*>(dl) = u4v{lo[0], lo[1], lo[2], lo[3]};
+      *reinterpret_cast<u4v*>(dh) = u4v{hi[0], hi[1], hi[2], hi[3]};
+    } else {
+      *reinterpret_cast<u2v*>(dl) = u2v{lo[0], lo[1]};
+      *reinterpret_cast<u2v*>(dh) = u2v{hi[0], hi[1]};
+    }
   };
 
-  h8 af[2][MI], bf[2][4];  // fragments of two 16-wide k-steps
+  h8 af[2][MI], bf[2][NJ];  // fragments of two 16-wide k-steps
   auto load_frags = [&](int buf, int ks, int fs) {
     const unsigned char* as = As + buf * PF_TILE_BYTES + wm * PF_ROW_BYTES;
     const unsigned char* bs = Bs + buf * PF_TILE_BYTES + wn * PF_ROW_BYTES;
@@ -214,14 +232,14 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
     for (int i = 0; i < MI; ++i)
       af[fs][i] = *reinterpret_cast<const h8*>(as + 32 * i * PF_ROW_BYTES + fa_off[ks ^ (2 * (i & 1))]);
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
       bf[fs][j] = *reinterpret_cast<const h8*>(bs + 32 * j * PF_ROW_BYTES + f_off[ks ^ (2 * (j & 1))]);
   };
   auto mfma_step = [&](int fs) {
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < NJ; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[fs][i], bf[fs][j], acc[i][j], 0, 0, 0);
   };
 
@@ -229,11 +247,12 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   // passes, during which the wave can issue about seven other instructions, so the other
   // work of the phase is dealt out evenly between the MFMAs: per MFMA pair `valu` VALU ops,
   // `dsr` LDS reads, `dsw` LDS writes and `vm` buffer loads.
+  constexpr int NPAIR = MI * NJ / 2 > 0 ? MI * NJ / 2 : 1;   // MFMA pairs per phase
   auto phase_schedule = [&](auto VALU, auto DSR, auto DSW, auto VM) {
     constexpr int valu = decltype(VALU)::value, dsr = decltype(DSR)::value;
     constexpr int dsw = decltype(DSW)::value, vm = decltype(VM)::value;
 #pragma unroll
-    for (int i = 0; i < 2 * MI; ++i) {
+    for (int i = 0; i < NPAIR; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       if (dsr) __builtin_amdgcn_sched_group_barrier(0x100, dsr, 0);
       if (vm) __builtin_amdgcn_sched_group_barrier(0x020, vm, 0);
@@ -247,12 +266,17 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
-  // per-MFMA-pair shares; the 128-row tile has half the MFMAs per phase for the same W work
-  using VA = std::integral_constant<int, 48 / (2 * MI)>;             // dequant VALU, phases 1 and 2
-  using VB = std::integral_constant<int, 96 / (2 * MI)>;             // phase 3
-  using DR = std::integral_constant<int, MI == 4 ? 1 : (MI == 1 ? 3 : 2)>;   // fragment reads
-  using DW1 = std::integral_constant<int, MI == 4 ? 1 : (MI == 3 ? 2 : (MI == 2 ? 3 : 4))>;  // LDS writes, phase 1 (X tile + byte 0)
-  using VM1 = std::integral_constant<int, MI == 2 ? 3 : (MI == 1 ? 6 : 2)>;   // W / zero / scale loads, phase 1
+  // per-MFMA-pair shares of the phase's other work (smaller tiles have fewer MFMAs per phase
+  // for the same W work; with eight waves a thread has half the W and X work)
+  constexpr auto cdiv = [](int a, int b) { return (a + b - 1) / b; };
+  using VA = std::integral_constant<int, cdiv(6 * RW, NPAIR)>;        // dequant VALU of one byte, phases 1 and 2
+  using VB = std::integral_constant<int, cdiv(12 * RW, NPAIR)>;       // two bytes, phase 3
+  using DR = std::integral_constant<int, cdiv(MI + NJ, NPAIR)>;       // fragment reads
+  using DW1 = std::integral_constant<int, (MI == 4 && NWV == 4) ? 1 : cdiv(AL + 2, NPAIR)>;  // X tile + byte 0
+  using DW2 = std::integral_constant<int, cdiv(2, NPAIR)>;
+  using DW3 = std::integral_constant<int, cdiv(4, NPAIR)>;
+  using VM1 = std::integral_constant<int, cdiv(RW + 2, NPAIR)>;       // W / zero / scale loads, phase 1
+  using VM2 = std::integral_constant<int, cdiv(AL, NPAIR)>;           // X loads, phase 2
 
   // One k-tile, PAR = kt & 1.  On entry: LDS buffer PAR holds tile kt and fragment set 0 its
   // first k-step; areg and W set PAR^1 hold tile kt + 1; W set PAR is free.  Tiles past the
@@ -275,7 +299,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
     load_frags(PAR, 2, 0);
     gload_a(kt2);
     dq_byte(PAR ^ 1, PAR ^ 1, I1{});
-    phase_schedule(VA{}, DR{}, I1{}, I1{});
+    phase_schedule(VA{}, DR{}, DW2{}, VM2{});
     __builtin_amdgcn_sched_barrier(0);
 
     // phase 3: bytes 2 and 3 of W(kt+1)
@@ -283,7 +307,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
     load_frags(PAR, 3, 1);
     dq_byte(PAR ^ 1, PAR ^ 1, I2{});
     dq_byte(PAR ^ 1, PAR ^ 1, I3{});
-    phase_schedule(VB{}, DR{}, I1{}, I0{});
+    phase_schedule(VB{}, DR{}, DW3{}, I0{});
     __builtin_amdgcn_sched_barrier(0);
 
     // every LDS write of tile kt + 1 is out and every read of tile kt has returned
@@ -325,12 +349,12 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < NJ; ++j)
 #pragma unroll
         for (int r = 0; r < 16; r += 4) {
-          const int q = ((i * 4 + j) * 16 + r) >> 2;
+          const int q = ((i * NJ + j) * 16 + r) >> 2;
           const f4 v = {acc[i][j][r], acc[i][j][r + 1], acc[i][j][r + 2], acc[i][j][r + 3]};
-          *reinterpret_cast<f4*>(mine + ((size_t)q * 256 + tid) * 4) = v;
+          *reinterpret_cast<f4*>(mine + ((size_t)q * NTH + tid) * 4) = v;
         }
     // summed and written out by awq_gemm_mfma_reduce_kernel, launched behind this kernel
     return;
@@ -341,7 +365,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       const int col = n0 + wn + 32 * j + col_l;
       if (col >= p.N) continue;
 #pragma unroll
@@ -353,12 +377,14 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_mfma_kernel(const MfmaGemmPar
 }
 
 // Sum of the split-K partial tiles.  Partial layout per (tile, part): [q][thread] groups of
-// four floats, q = (i * 4 + j) * 4 + r / 4 over the MI x 4 accumulator tiles of the producing
-// thread.  One workgroup takes four q of one tile; parts are added in index order.
-template <int MI>
-__global__ __launch_bounds__(256) void awq_gemm_mfma_reduce_kernel(const MfmaGemmParams p) {
+// four floats, q = (i * NJ + j) * 4 + r / 4 over the MI x NJ accumulator tiles of the producing
+// thread (same thread count and wave arrangement as the producer).  One workgroup takes four
+// q of one tile; parts are added in index order.
+template <int MI, int NWV = 4>
+__global__ __launch_bounds__(64 * NWV) void awq_gemm_mfma_reduce_kernel(const MfmaGemmParams p) {
   constexpr int QPW = 4;
-  constexpr int QT = 16 * MI;
+  constexpr int NJ = 16 / NWV, NTH = 64 * NWV;
+  constexpr int QT = 4 * MI * NJ;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int tl = blockIdx.x / (QT / QPW);
   const int q0 = (blockIdx.x % (QT / QPW)) * QPW;
@@ -369,7 +395,7 @@ __global__ __launch_bounds__(256) void awq_gemm_mfma_reduce_kernel(const MfmaGem
   const int mt_i = first_m + (nid % gsize) % gm;
   const int nt_i = (nid % gsize) / gm;
   const int m0 = mt_i * (64 * MI), n0 = nt_i * PF_BN;
-  const int wm = (wave >> 1) * (32 * MI), wn = (wave & 1) * 128;
+  const int wm = (wave / (NWV / 2)) * (32 * MI), wn = (wave % (NWV / 2)) * (32 * NJ);
   const int col_l = lane & 31, row_l = 4 * (lane >> 5);
   const float* tile_base = p.sk_part + (size_t)tl * p.sk_split * PF_SK_SLOT_FLOATS;
   f4 v[QPW];
@@ -380,7 +406,7 @@ __global__ __launch_bounds__(256) void awq_gemm_mfma_reduce_kernel(const MfmaGem
 #pragma unroll
     for (int u = 0; u < QPW; ++u)
       t[u] = *reinterpret_cast<const f4*>(tile_base + (size_t)s * PF_SK_SLOT_FLOATS +
-                                          ((size_t)(q0 + u) * 256 + tid) * 4);
+                                          ((size_t)(q0 + u) * NTH + tid) * 4);
 #pragma unroll
     for (int u = 0; u < QPW; ++u) v[u] += t[u];
   }
@@ -388,8 +414,8 @@ __global__ __launch_bounds__(256) void awq_gemm_mfma_reduce_kernel(const MfmaGem
   for (int u = 0; u < QPW; ++u) {
     const int q = q0 + u;
     const int ij = q >> 2, r = (q & 3) * 4;
-    const int col = n0 + wn + 32 * (ij & 3) + col_l;
-    const int row = m0 + wm + 32 * (ij >> 2) + 8 * (r >> 2) + row_l;
+    const int col = n0 + wn + 32 * (ij % NJ) + col_l;
+    const int row = m0 + wm + 32 * (ij / NJ) + 8 * (r >> 2) + row_l;
     if (col < p.N) {
 #pragma unroll
       for (int e = 0; e < 4; ++e)

@@ -118,9 +118,6 @@ struct GemvWave {
   NibbleMasks nm;
 
   __device__ __forceinline__ void issue(int d, int ks) {
-#ifdef AWQMI_LAB_STEP_MASK   // lab only: alias all steps onto a few, so loads hit in L2
-    ks &= AWQMI_LAB_STEP_MASK;
-#endif
     const char* rowbase = reinterpret_cast<const char*>(qw_u) + (size_t)ks * 32 * NW * 4;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
@@ -171,16 +168,6 @@ struct GemvWave {
   }
 
   __device__ __forceinline__ void compute(int d, bool first) {
-#ifdef AWQMI_LAB_NO_COMPUTE    // lab only: consume the loads without the unpack / MFMA work
-    u4v x = a[d][0];
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-      for (int w = 0; w < WPL; ++w) x[0] ^= WordVec<WPL>::get(q[d][i], w);
-    acc[0][0] += __builtin_bit_cast(f4, x);
-    (void)first;
-    return;
-#endif
     // this lane's share of sum_k x_k
     const h2 ones = {(half_t)1.f, (half_t)1.f};
 #pragma unroll
@@ -206,9 +193,6 @@ struct GemvWave {
 
   // end of a group: zero-point MFMA, then acc += s * accg
   __device__ __forceinline__ void flush() {
-#ifdef AWQMI_LAB_NO_COMPUTE
-    return;
-#endif
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       // xsum as three fp16 pieces (33 significant bits) in k-slots 0..2 against -z there
@@ -400,9 +384,6 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
   const int c_begin = (int)(pw * nchunks / parts);
   const int c_end = (int)((pw + 1) * nchunks / parts);
   w.run(c_begin, c_end);
-#if defined(AWQMI_LAB_EPI) && AWQMI_LAB_EPI == 4
-  if (p.M != 12345) return;
-#endif
 
   const int rows_total = MOE ? s_rows : p.M;
   const size_t tile = (size_t)blk * p.ncb + cb;
@@ -492,9 +473,6 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
         }
     }
     __syncthreads();
-#if defined(AWQMI_LAB_EPI) && AWQMI_LAB_EPI == 3
-    if (p.M != 12345) return;
-#endif
     if (split) {
       // fp32 partial tile of this workgroup.  Partials and the arrival counter go through
       // device-coherent accesses (they bypass the per-XCD L2 for other XCDs' data) instead of
@@ -514,9 +492,6 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
     __syncthreads();
   }
   if (!split) return;
-#if defined(AWQMI_LAB_EPI) && AWQMI_LAB_EPI == 2
-  if (p.M != 12345) return;
-#endif
 
   // Ordering: every store of this workgroup has completed (vmcnt 0, then the barrier)
   // before its arrival is counted; whoever arrives last sums all partials in fixed order.
@@ -525,9 +500,6 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
   if (tid == 0) s_last = (atomicAdd(p.cnt + tile, 1) == p.split_k - 1);
   __syncthreads();
   if (!s_last) return;
-#if defined(AWQMI_LAB_EPI) && AWQMI_LAB_EPI == 1
-  if (p.M != 12345) { if (tid == 0) __hip_atomic_store(p.cnt + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); return; }
-#endif
   const size_t sstride = ntiles * MB * TILE_F;
   // U pairs per thread x 8 parts per batch: 8 * U independent 8-byte loads in flight; parts
   // are added in index order whatever the arrival order was.  Out-of-range slots read a valid
