@@ -160,3 +160,36 @@ def test_fused_call_graph_replay(sba, gpu):
             sba.awq_gemm(c.x, c.w13[0][0], c.w13[1][0], c.w13[2][0], 0)   # unrelated eager work
             torch.cuda.synchronize()
     torch.cuda.current_stream().wait_stream(s)
+
+
+def _dense_expert_reference(sba, c, gpu, T, H, E, topk, I):
+    """Every expert evaluated densely with the dequantize kernel + a library matmul."""
+    w, ids = sba.topk_softmax(c.logits, topk, True)
+    ref = torch.zeros((T, H), dtype=torch.float32, device=gpu)
+    for e in range(E):
+        tok, slot = torch.nonzero(ids == e, as_tuple=True)
+        if tok.numel() == 0:
+            continue
+        W13 = sba.awq_dequantize(c.w13[0][e], c.w13[1][e], c.w13[2][e]).float()
+        W2 = sba.awq_dequantize(c.w2[0][e], c.w2[1][e], c.w2[2][e]).float()
+        h = (c.x[tok].float() @ W13).half().float()
+        a = (torch.nn.functional.silu(h[:, :I]) * h[:, I:]).half().float()
+        o = ((a @ W2) * w[tok, slot][:, None]).half().float()
+        ref.index_add_(0, tok, o)
+    return ref
+
+
+@pytest.mark.parametrize("T,H,E,topk,I", [
+    (8192, 512, 16, 4, 256),     # more (block, column block) tiles than arrival counters: split-K is switched off
+    (300, 384, 60, 3, 128),      # expert count that is no multiple of 64, odd top-k, ragged last blocks
+    (40, 256, 8, 1, 384),        # top-1, K of the second GEMM = 3 chunks (no column-block pairing)
+    (64, 256, 200, 8, 256),      # most experts idle
+])
+def test_moe_odd_shapes_vs_dense_expert_path(sba, gpu, T, H, E, topk, I):
+    c = sba.workloads.make_moe_case(T, H, E, topk, I, 128, seed=T + E).to(gpu)
+    y = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True)
+    ref = _dense_expert_reference(sba, c, gpu, T, H, E, topk, I)
+    err = float((y.float() - ref).norm() / ref.norm())
+    print(f"[moe odd T={T} E={E} topk={topk}] rel_fro={err:.2e}", flush=True)
+    assert err <= TOL
+    assert torch.equal(y, sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True))
