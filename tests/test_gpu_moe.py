@@ -180,7 +180,7 @@ def _dense_expert_reference(sba, c, gpu, T, H, E, topk, I):
 
 
 @pytest.mark.parametrize("T,H,E,topk,I", [
-    (8192, 512, 16, 4, 256),     # more (block, column block) tiles than arrival counters: split-K is switched off
+    (8192, 2048, 32, 8, 768),    # more (block, column block) tiles than arrival counters: split-K is switched off
     (300, 384, 60, 3, 128),      # expert count that is no multiple of 64, odd top-k, ragged last blocks
     (40, 256, 8, 1, 384),        # top-1, K of the second GEMM = 3 chunks (no column-block pairing)
     (64, 256, 200, 8, 256),      # most experts idle
