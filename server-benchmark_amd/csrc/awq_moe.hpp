@@ -69,9 +69,10 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __re
 // Single workgroup of 16 waves.  Dynamic LDS: cnt[16][E] + padded[E] + start[E].
 // Wave w owns the contiguous slice [w*seg, (w+1)*seg) of the flat slot list, so placing
 // slices in wave order and slots in index order inside a slice gives a stable sort.  Inside a
-// batch of 64 slots a lane's rank among equal expert ids is a count over lower lanes (64
-// scalar broadcasts, no LDS round trips); the running position per (wave, expert) lives in
-// LDS and is bumped by one LDS atomic per slot after all lanes of the batch have read it.
+// batch of 64 slots a lane's rank among equal expert ids is the number of lower lanes with
+// the same id (a lane mask built from one ballot per id bit, no LDS round trips); the running
+// position per (wave, expert) lives in LDS and is bumped by one LDS atomic per slot after all
+// lanes of the batch have read it.
 constexpr int MOE_ALIGN_WAVES = 16;
 __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int n, int E,
                                                          int tile_m, int cap,
@@ -91,9 +92,32 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
 
   const int seg = ((n + NWV * 64 - 1) / (NWV * 64)) * 64;
   const int sb = wave * seg, se = min(n, sb + seg);
-  for (int i = sb + lane; i < se; i += 64) {
-    const int e = ids[i];
+  // ids are read eight batches of 64 at a time (eight loads in flight instead of one
+  // dependent load per batch); the first eight batches stay in registers for the second pass
+  constexpr int NB = 8;
+  int first[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    const int i = sb + 64 * b + lane;
+    first[b] = i < se ? ids[i] : -1;
+  }
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    const int e = first[b];
     if (e >= 0 && e < E) atomicAdd(&cnt[wave * E + e], 1);
+  }
+  for (int c0 = sb + 64 * NB; c0 < se; c0 += 64 * NB) {
+    int more[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int i = c0 + 64 * b + lane;
+      more[b] = i < se ? ids[i] : -1;
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int e = more[b];
+      if (e >= 0 && e < E) atomicAdd(&cnt[wave * E + e], 1);
+    }
   }
   __syncthreads();
 
@@ -136,22 +160,39 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
   for (int i = total / tile_m + tid; i < cap / tile_m; i += 1024) expert_ids[i] = -1;
   __syncthreads();
 
-  for (int i0 = sb; i0 < se; i0 += 64) {
-    const int i = i0 + lane;
-    int e = i < se ? ids[i] : -1;
+  const int nbits = 32 - __builtin_clz(max(E - 1, 1));
+  auto place = [&](int i, int e) {
     const bool valid = e >= 0 && e < E;
-    if (!valid) e = -1 - lane;     // never equal to another lane's id
-    int rank = 0;
-    for (int l = 0; l < 63; ++l) {
-      const int el = __builtin_amdgcn_readlane(e, l);
-      rank += (el == e && l < lane) ? 1 : 0;
+    // lanes of the batch that hold the same expert id: one ballot per id bit
+    unsigned long long same = __ballot(valid);
+    for (int b = 0; b < nbits; ++b) {
+      const bool bit = (e >> b) & 1;
+      const unsigned long long bal = __ballot(bit);
+      same &= bit ? bal : ~bal;
     }
+    const int rank = __popcll(same & ((1ull << lane) - 1ull));   // equal ids in lower lanes
     int base = 0;
     if (valid) base = cnt[wave * E + e];
     __builtin_amdgcn_wave_barrier();
     if (valid) {
       sorted[base + rank] = i;
       atomicAdd(&cnt[wave * E + e], 1);
+    }
+  };
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    if (sb + 64 * b < se) place(sb + 64 * b + lane, first[b]);     // wave-uniform condition
+  }
+  for (int c0 = sb + 64 * NB; c0 < se; c0 += 64 * NB) {
+    int more[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int i = c0 + 64 * b + lane;
+      more[b] = i < se ? ids[i] : -1;
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      if (c0 + 64 * b < se) place(c0 + 64 * b + lane, more[b]);
     }
   }
 }
