@@ -4,6 +4,7 @@
 // from the thread-local last HIP error and the development variant switch.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <type_traits>
 
@@ -473,8 +474,11 @@ int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales
   if (variant >= 0 && ((variant >> 2) & 7)) p.grp = 1 << (((variant >> 2) & 7) - 1);
   // few chunks of K and no split across workgroups: two column blocks per workgroup, two
   // waves each (three chunks per wave at K = 768 instead of 2 / 2 / 1 / 1)
+  // -- as long as the paired launch still fills the chip (blocks that will run: one per expert
+  // touched or per 16 slots, whichever is more)
+  const long long live_blocks = std::max<long long>((n_slots + 15) / 16, std::min(n_slots, E));
   const bool pair_cols = tile_m == 16 && wpl == 2 && split == 1 && K / 128 <= 8 && (K / 128) % 2 == 0 &&
-                         !(variant >= 0 && (variant & 64));
+                         live_blocks * ((ncb + 1) / 2) >= 256 && !(variant >= 0 && (variant & 64));
   const int ncg = pair_cols ? (ncb + 1) / 2 : ncb;
   // runs of grp slots, dealt to the 8 XCDs in turn; the last deal may be partial
   const long long runs = (long long)(nblk / p.grp) * ncg * split;
