@@ -244,3 +244,23 @@ def test_linear_method_apply(sba, gpu):
     assert y.shape == (2, 3, 256)
     ref = awq_ref.gemm_wide(x, qw, s, qz, 128) + bias.cpu().numpy().astype(np.float64)
     assert awq_ref.rel_frobenius(y.reshape(6, 256).cpu().numpy(), ref) <= TOL
+
+
+def test_gemm_random_shapes_across_dispatch_boundaries(sba, gpu):
+    """Seeded random (M, K, N, G) around every boundary of the kernel choice (16 / 32 / 48 / 64 /
+    128 / 192 / 256 rows, odd word counts, ragged tiles, K-split on and off), against the oracle."""
+    rng = np.random.default_rng(2024)
+    ms = [1, 2, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 100, 127, 128, 129, 191, 192, 193, 255, 256, 257, 300]
+    worst = 0.0
+    for case in range(40):
+        M = int(ms[case % len(ms)]) if case < len(ms) else int(rng.integers(1, 320))
+        G = int(rng.choice([32, 64, 128, 256]))
+        K = int(rng.integers(1, 9)) * 256
+        N = int(rng.integers(1, 150)) * 8
+        x, qw, s, qz = _np_case(M, K, N, G, seed=1000 + case)
+        y = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), 0).cpu().numpy()
+        ref = awq_ref.gemm_wide(x, qw, s, qz, G)
+        err = awq_ref.rel_frobenius(y, ref)
+        assert err <= TOL, f"M={M} K={K} N={N} G={G}: rel_fro={err:.3e}"
+        worst = max(worst, err)
+    print(f"[random shapes] worst rel_fro={worst:.2e}", flush=True)
