@@ -102,7 +102,7 @@ inline bool skinny_rows(int M, int N) {
 
 // Work split of the MFMA kernel: whole rounds of 256 tiles run one workgroup per tile; a
 // last round of fewer than 129 tiles (and any launch that small) is split in K over
-// floor(256 / tiles) workgroups per tile (at most 8, at least 8 k-tiles each).
+// floor(256 / tiles) workgroups per tile (at most 8, at least 4 k-tiles each).
 // The MFMA kernel addresses X through 32-bit buffer offsets: calls with more than 4 GiB of
 // activations run as consecutive row slabs (multiples of 256 rows).
 inline int mfma_slab_rows(int M, int K) {
@@ -120,7 +120,7 @@ MfmaPlan plan_mfma(int M, int K, int N) {
   if (rem == 0) return pl;
   int c = 256 / rem;
   if (c > 8) c = 8;
-  while (c > 1 && KT / c < 8) --c;
+  while (c > 1 && KT / c < 4) --c;
   if (c < 2) return pl;
   pl.dp_tiles = tiles - rem;
   pl.sk_tiles = rem;
