@@ -82,12 +82,12 @@ inline size_t gemv_partial_bytes(int N, int split, long long blocks_z, int tile_
   return (size_t)split * (size_t)blocks_z * tile_m * npad * sizeof(float);
 }
 
-template <int WPL, int MB, bool MOE, int RING = 4, int KW = 4>
+template <int WPL, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false>
 void launch_gemv(const GemvParams& p, dim3 grid, hipStream_t st) {
-  if (p.G == 32) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MB, MOE, RING, KW>), grid, dim3(256), 0, st, p);
-  else if (p.G == 64) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MB, MOE, RING, KW>), grid, dim3(256), 0, st, p);
-  else if (p.G == 128) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MB, MOE, RING, KW>), grid, dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MB, MOE, RING, KW>), grid, dim3(256), 0, st, p);
+  if (p.G == 32) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MB, MOE, RING, KW, ACT>), grid, dim3(256), 0, st, p);
+  else if (p.G == 64) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MB, MOE, RING, KW, ACT>), grid, dim3(256), 0, st, p);
+  else if (p.G == 128) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MB, MOE, RING, KW, ACT>), grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MB, MOE, RING, KW, ACT>), grid, dim3(256), 0, st, p);
 }
 
 // rows the skinny kernel takes in one awq_gemm call (passes of up to 32 rows)
@@ -249,7 +249,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     p.cnt = reinterpret_cast<int*>(workspace);
     p.part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
                        : nullptr;
-    p.K = K; p.N = N; p.NW = NW; p.G = G;
+    p.K = K; p.N = N; p.NW = NW; p.G = G; p.ldy = N;
     p.split_k = split; p.ncb = ncb;
     const dim3 grid(ncb, split, 1);
     // passes of up to 32 rows; each pass streams the weights once
@@ -424,11 +424,38 @@ size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int spli
   return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, pl.split, pl.nblk, tile_m);
 }
 
+// Can the w13 GEMM of a block write silu(gate) * up itself?  Needs the paired-column launch
+// (two column blocks per workgroup: the gate block and its up block), i.e. no split across
+// workgroups, an even chunk count, [gate | up] halves that are whole column blocks, and
+// enough blocks that the halved workgroup count still fills the chip.
+static bool moe_can_fuse_act(int n_slots, int E, int K, int N) {
+  const MoePlan pl = moe_plan(n_slots, E, K, N, 16, 0);
+  const long long live_blocks = std::max<long long>((n_slots + 15) / 16, std::min(n_slots, E));
+  return pl.wpl == 2 && pl.split == 1 && K % 128 == 0 && (K / 128) % 2 == 0 && N % 512 == 0 &&
+         live_blocks * (pl.ncb / 2) >= 256;
+}
+
+static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                         void* y, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                         const int32_t* num_tokens_post_padded, const float* topk_weights, int n_slots,
+                         int a_row_div, int tile_m, int E, int K, int N, int group, int split_k,
+                         void* workspace, size_t workspace_bytes, void* stream, bool fuse_act);
+
 int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
                        void* y, const int32_t* sorted_token_ids, const int32_t* expert_ids,
                        const int32_t* num_tokens_post_padded, const float* topk_weights, int n_slots,
                        int a_row_div, int tile_m, int E, int K, int N, int group, int split_k,
                        void* workspace, size_t workspace_bytes, void* stream) {
+  return moe_gemm_impl(x, qweight, scales, qzeros, y, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                       topk_weights, n_slots, a_row_div, tile_m, E, K, N, group, split_k, workspace,
+                       workspace_bytes, stream, false);
+}
+
+static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                         void* y, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                         const int32_t* num_tokens_post_padded, const float* topk_weights, int n_slots,
+                         int a_row_div, int tile_m, int E, int K, int N, int group, int split_k,
+                         void* workspace, size_t workspace_bytes, void* stream, bool fuse_act) {
   if (!x || !qweight || !scales || !qzeros || !y || !sorted_token_ids || !expert_ids ||
       !num_tokens_post_padded)
     return AWQMI_NULL_POINTER;
@@ -468,6 +495,7 @@ int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales
   p.topk_w = topk_weights; p.n_slots = n_slots; p.a_row_div = a_row_div; p.tile_m = tile_m;
   p.w_stride = (long long)K * NW; p.s_stride = (long long)(K / G) * N; p.z_stride = (long long)(K / G) * NW;
   p.nblk = nblk;
+  p.ldy = fuse_act ? N / 2 : N;
   const int variant = g_gemv_variant.load(std::memory_order_relaxed);
   // group blocks by XCD once experts average two blocks or more
   p.grp = (long long)n_slots >= 2LL * tile_m * E ? 8 : 1;
@@ -479,12 +507,15 @@ int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales
   const long long live_blocks = std::max<long long>((n_slots + 15) / 16, std::min(n_slots, E));
   const bool pair_cols = tile_m == 16 && wpl == 2 && split == 1 && K / 128 <= 8 && (K / 128) % 2 == 0 &&
                          live_blocks * ((ncb + 1) / 2) >= 256 && !(variant >= 0 && (variant & 64));
-  const int ncg = pair_cols ? (ncb + 1) / 2 : ncb;
+  if (fuse_act && (split != 1 || wpl != 2 || tile_m != 16 || ncb % 2 != 0 || (K / 128) % 2 != 0))
+    return AWQMI_BAD_ARGUMENT;
+  const int ncg = fuse_act ? ncb / 2 : (pair_cols ? (ncb + 1) / 2 : ncb);
   // runs of grp slots, dealt to the 8 XCDs in turn; the last deal may be partial
   const long long runs = (long long)(nblk / p.grp) * ncg * split;
   const dim3 grid((unsigned)((runs + 7) / 8 * 8 * p.grp));
   hipStream_t st = (hipStream_t)stream;
-  if (tile_m == 32) launch_gemv<2, 2, true>(p, grid, st);
+  if (fuse_act) launch_gemv<2, 1, true, 2, 2, true>(p, grid, st);
+  else if (tile_m == 32) launch_gemv<2, 2, true>(p, grid, st);
   else if (wpl == 2 && variant >= 0 && (variant & 2)) launch_gemv<2, 1, true, 4>(p, grid, st);
   else if (pair_cols) launch_gemv<2, 1, true, 2, 2>(p, grid, st);
   else if (wpl == 2) launch_gemv<2, 1, true, 2>(p, grid, st);
@@ -577,11 +608,21 @@ int awqmi_fused_moe_f16(const void* hidden, const float* router_logits, const in
   if (st) return st;
   st = awqmi_moe_align(ids, L.n_slots, E, 16, sorted, experts, npp, stream);
   if (st) return st;
-  st = awqmi_moe_gemm_f16(hidden, w13_q, w13_s, w13_z, h13, sorted, experts, npp, nullptr, L.n_slots, topk,
-                          16, E, H, 2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream);
-  if (st) return st;
-  st = awqmi_silu_and_mul_f16(h13, act, L.n_slots, inter, stream);
-  if (st) return st;
+  const int Gn = norm_group(H, group);
+  if (gemv_tiled_ok(H, Gn) && moe_can_fuse_act(L.n_slots, E, H, 2 * inter) &&
+      !(g_gemv_variant.load(std::memory_order_relaxed) >= 0 &&
+        (g_gemv_variant.load(std::memory_order_relaxed) & 1024))) {
+    // the w13 GEMM writes silu(gate) * up itself
+    st = moe_gemm_impl(hidden, w13_q, w13_s, w13_z, act, sorted, experts, npp, nullptr, L.n_slots, topk, 16, E, H,
+                       2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream, true);
+    if (st) return st;
+  } else {
+    st = awqmi_moe_gemm_f16(hidden, w13_q, w13_s, w13_z, h13, sorted, experts, npp, nullptr, L.n_slots, topk,
+                            16, E, H, 2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream);
+    if (st) return st;
+    st = awqmi_silu_and_mul_f16(h13, act, L.n_slots, inter, stream);
+    if (st) return st;
+  }
   st = awqmi_moe_gemm_f16(act, w2_q, w2_s, w2_z, o, sorted, experts, npp, wts, L.n_slots, 1, 16, E, inter, H,
                           group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream);
   if (st) return st;

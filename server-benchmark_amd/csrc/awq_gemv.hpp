@@ -39,6 +39,7 @@ struct GemvParams {
   int n_slots;
   int a_row_div;
   int tile_m;   // rows per sorted-token block: 16 * MB
+  int ldy;      // elements between output rows (N, or N / 2 when the activation is fused)
   int nblk;     // sorted-token blocks covered by the launch (a multiple of grp)
   int grp;      // sorted-token blocks per XCD run
   long long w_stride, s_stride, z_stride;  // elements per expert
@@ -299,8 +300,12 @@ struct GemvWave {
 // workgroup then covers two neighbouring column blocks with two waves each, which keeps the
 // waves' ranges long and even when K is only a few chunks; launches with KW = 2 do not split K
 // across workgroups).
-template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4>
+// ACT (with KW = 2): the weight columns are [gate | up]; the workgroup takes a gate column
+// block and the up column block N / 2 columns further, and writes silu(gate) * up (both rounded
+// to fp16 first, as the unfused path stores them) to a [.., N / 2] output.
+template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false>
 __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
+  static_assert(!ACT || (KW == 2 && MB == 1), "fused activation pairs two column blocks");
   constexpr int CW = 4 / KW;       // column blocks per workgroup
   constexpr int NT = 8 * WPL;
   constexpr int CB = 128 * WPL;
@@ -322,7 +327,7 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
     const int B = p.grp;
     const int lin = blockIdx.x, xcd = lin & 7, slot = lin >> 3;
     const int g = (slot / B) * 8 + xcd;            // run index: (block group, column block, part)
-    const int ncbs = ((p.ncb + CW - 1) / CW) * p.split_k;
+    const int ncbs = (ACT ? p.ncb / 2 : (p.ncb + CW - 1) / CW) * p.split_k;
     const int bg = g / ncbs, cbs = g % ncbs;
     blk = bg * B + slot % B;
     cb = cbs / p.split_k;          // column group of the workgroup (a column block when CW = 1)
@@ -350,7 +355,7 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
   // Lanes past the last word column / past the last row read valid memory of column block 0
   // / row 0 instead; their B column (resp. A row) only feeds outputs that are never stored.
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-  const int cbw = cb * CW + wave_u / KW;     // this wave's column block
+  const int cbw = ACT ? cb + (wave_u / KW) * (p.ncb / 2) : cb * CW + wave_u / KW;   // this wave's column block
   int wc = cbw * (16 * WPL) + WPL * j;
   if (wc >= p.NW) wc = 0;
 
@@ -420,7 +425,27 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
       h8 o;
 #pragma unroll
       for (int c = 0; c < 8; ++c) o[c] = (half_t)v[c];
-      *reinterpret_cast<h8*>(p.y + orow * p.N + col) = o;
+      *reinterpret_cast<h8*>(p.y + orow * p.ldy + col) = o;
+    }
+  };
+  // gate tile in red[0], up tile in red[1] -> silu(gate) * up, 16 bytes per thread
+  auto emit_act = [&](int rows) {
+    constexpr int WPB = 16 * WPL;
+    for (int it = tid; it < rows * WPB; it += 256) {
+      const int m = it / WPB, wl = it % WPB;
+      const int jj = wl / WPL, ww = wl % WPL;
+      const int col = cb * CB + wl * 8;
+      const int sid = s_sid[m];
+      if (sid >= p.n_slots) continue;
+      h8 o;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const int t = ww * 8 + awq_nibble_of_col(c);
+        const float gv = (float)(half_t)red[0][m][t * 16 + jj];
+        const float uv = (float)(half_t)red[1][m][t * 16 + jj];
+        o[c] = (half_t)(gv / (1.f + __expf(-gv)) * uv);
+      }
+      *reinterpret_cast<h8*>(p.y + (size_t)sid * p.ldy + col) = o;
     }
   };
 
@@ -448,8 +473,12 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
           }
       }
       __syncthreads();
-      emit(mb, rows, false, 0, cb * 2);
-      if (cb * 2 + 1 < p.ncb) emit(mb, rows, false, 1, cb * 2 + 1);
+      if (ACT) {
+        emit_act(rows);
+      } else {
+        emit(mb, rows, false, 0, cb * 2);
+        if (cb * 2 + 1 < p.ncb) emit(mb, rows, false, 1, cb * 2 + 1);
+      }
       __syncthreads();
       continue;
     }

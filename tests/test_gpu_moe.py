@@ -193,3 +193,20 @@ def test_moe_odd_shapes_vs_dense_expert_path(sba, gpu, T, H, E, topk, I):
     print(f"[moe odd T={T} E={E} topk={topk}] rel_fro={err:.2e}", flush=True)
     assert err <= TOL
     assert torch.equal(y, sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True))
+
+
+@pytest.mark.parametrize("T", [128, 512])
+def test_fused_activation_agrees_with_step_by_step(sba, gpu, T):
+    """Block sizes at which the w13 GEMM of the one-call path writes silu(gate) * up itself.  Its
+    two waves per column block add K in another order than the four of the separate-kernel
+    path, so the two agree to fp32 summation order (a few last-bit differences after the fp16
+    roundings), not bit for bit; both must meet the tolerance against the dense expert path."""
+    c = sba.workloads.make_moe_case(T, 2048, 128, 8, 768, 128, seed=300 + T).to(gpu)
+    step = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 8, True, block_size=16)
+    one = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 8, True)
+    d = float((one.float() - step.float()).norm() / step.float().norm())
+    print(f"[moe fused act T={T}] vs step-by-step rel_fro={d:.2e}", flush=True)
+    assert d <= 2e-4
+    ref = _dense_expert_reference(sba, c, gpu, T, 2048, 128, 8, 768)
+    assert float((one.float() - ref).norm() / ref.norm()) <= TOL
+    assert torch.equal(one, sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 8, True))
