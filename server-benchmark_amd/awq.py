@@ -55,6 +55,17 @@ class AWQConfig:
         return ["quant_config.json", "quantize_config.json"]
 
     @classmethod
+    def get_min_capability(cls) -> int:
+        """vLLM asks every quantisation config for a minimum CUDA compute capability; on a
+        ROCm build the check is a formality, so report the value vLLM's AWQ config reports."""
+        return 75
+
+    @staticmethod
+    def get_scaled_act_names():
+        """Activations AWQ checkpoints may carry an input scale for (same list as vLLM's)."""
+        return ["gelu", "gelu_fast", "gelu_new", "gelu_pytorch_tanh"]
+
+    @classmethod
     def from_config(cls, config: dict) -> "AWQConfig":
         bits = _first_key(config, ("w_bit", "bits"))
         group = _first_key(config, ("q_group_size", "group_size"))

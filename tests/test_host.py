@@ -137,6 +137,13 @@ def test_awq_config_aliases(sba, cfg, want):
     assert torch.float16 in c.get_supported_act_dtypes()
 
 
+def test_awq_config_static_surface(sba):
+    cfg = sba.AWQConfig
+    assert cfg.get_name() == "awq" and cfg.get_min_capability() == 75
+    assert cfg.get_config_filenames() == ["quant_config.json", "quantize_config.json"]
+    assert "gelu" in cfg.get_scaled_act_names()
+
+
 def test_awq_config_rejects(sba):
     with pytest.raises(ValueError):
         sba.AWQConfig.from_config({"bits": 8, "group_size": 128, "zero_point": True})
