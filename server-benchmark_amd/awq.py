@@ -182,7 +182,23 @@ class AWQMoEMethod:
             setattr(layer, name, Parameter(t.data.contiguous(), requires_grad=False))
 
     def apply(self, layer: torch.nn.Module, x: torch.Tensor, router_logits: torch.Tensor, top_k: int,
-              renormalize: bool = True) -> torch.Tensor:
+              renormalize: bool = True, use_grouped_topk: bool = False, topk_group: Optional[int] = None,
+              num_expert_group: Optional[int] = None, global_num_experts: int = -1, expert_map=None,
+              custom_routing_function=None, scoring_func: str = "softmax", e_score_correction_bias=None,
+              activation: str = "silu", **unused) -> torch.Tensor:
+        """Same keyword surface as vLLM's fused-MoE methods.  Supported: softmax scoring, plain
+        top-k (optionally renormalised), SiLU, all experts local; anything else is refused
+        rather than silently computed differently."""
+        if use_grouped_topk or topk_group or num_expert_group:
+            raise NotImplementedError("grouped top-k routing is not implemented")
+        if custom_routing_function is not None or e_score_correction_bias is not None:
+            raise NotImplementedError("custom routing / score correction bias is not implemented")
+        if scoring_func != "softmax":
+            raise NotImplementedError(f"scoring function {scoring_func!r} is not implemented (softmax only)")
+        if activation != "silu":
+            raise NotImplementedError(f"activation {activation!r} is not implemented (silu only)")
+        if expert_map is not None or (global_num_experts not in (-1, layer.w13_qweight.shape[0])):
+            raise NotImplementedError("expert parallelism (expert_map / global_num_experts) is not implemented")
         shape = x.shape
         x2 = x.reshape(-1, shape[-1]).contiguous()
         out = ops.fused_moe_awq(x2, (layer.w13_qweight, layer.w13_scales, layer.w13_qzeros),

@@ -193,6 +193,18 @@ def test_moe_method_create_weights(sba):
 
 # ------------------------------------------------------------------ workloads
 
+def test_moe_method_refuses_unsupported_routing(sba):
+    m = sba.AWQMoEMethod(sba.AWQConfig(4, 128, True))
+    layer = torch.nn.Module()
+    m.create_weights(layer, 4, 256, 128, torch.float16)
+    x, lg = torch.zeros((2, 256), dtype=torch.float16), torch.zeros((2, 4))
+    for kw in (dict(use_grouped_topk=True), dict(scoring_func="sigmoid"), dict(activation="gelu"),
+               dict(expert_map=torch.arange(4)), dict(global_num_experts=8),
+               dict(custom_routing_function=lambda *a: None)):
+        with pytest.raises(NotImplementedError):
+            m.apply(layer, x, lg, 2, True, **kw)
+
+
 def test_workload_shapes_and_bytes(sba):
     w = sba.workloads
     c = w.config0()
