@@ -89,6 +89,15 @@ int awqmi_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales
 int awqmi_moe_topk_softmax_f32(const float* logits, int T, int E, int topk, int renormalize,
                                int32_t* topk_ids, float* topk_weights, void* stream);
 
+/* Router with the scoring variants of the MoE checkpoints the harness serves
+ * (reference config.yaml:36,47,51,134): scoring 0 = softmax (as above; score_bias must be
+ * null), scoring 1 = sigmoid: score = sigmoid(logit), experts are chosen by
+ * score + score_bias[e] (score_bias fp32 [E] or null), the weight is the score.  Weights are
+ * optionally renormalised over the chosen experts, then multiplied by `scale` (a routed
+ * scaling factor; 1 for none).  Ties go to the lowest expert id. */
+int awqmi_moe_topk_f32(const float* logits, const float* score_bias, int T, int E, int topk, int scoring,
+                       int renormalize, float scale, int32_t* topk_ids, float* topk_weights, void* stream);
+
 /* Capacity (entries) of sorted_token_ids for n = T*topk routed slots; expert_ids needs
  * capacity / tile_m entries. */
 size_t awqmi_moe_align_capacity(int n_slots, int E, int tile_m);

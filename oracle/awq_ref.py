@@ -103,6 +103,23 @@ def topk_softmax(logits: np.ndarray, topk: int, renormalize: bool = True):
     return order.astype(np.int32), w.astype(np.float32)
 
 
+def topk_sigmoid(logits: np.ndarray, topk: int, renormalize: bool = True, bias=None, scale: float = 1.0):
+    """score = sigmoid(logit); experts chosen by score + bias (ties: lowest id), weighted by the
+    score, optionally renormalised over the chosen ones, times scale.  (The routing of
+    sigmoid-scored MoE checkpoints with a score-correction bias and one expert group.)"""
+    lg = np.asarray(logits, np.float32).astype(np.float64)
+    score = 1.0 / (1.0 + np.exp(-lg))
+    # the device adds the bias in fp32 to an fp32 score: choose on the same values
+    key = score.astype(np.float32)
+    if bias is not None:
+        key = key + np.asarray(bias, np.float32)[None, :]
+    order = np.argsort(-key.astype(np.float64), axis=-1, kind="stable")[:, :topk]
+    w = np.take_along_axis(score, order, axis=-1)
+    if renormalize:
+        w = w / w.sum(axis=-1, keepdims=True)
+    return order.astype(np.int32), (w * scale).astype(np.float32)
+
+
 def moe_align(topk_ids: np.ndarray, num_experts: int, tile_m: int):
     """Stable sort of flat (token, slot) indices by expert, each expert's run padded to a
     multiple of tile_m with the sentinel T*topk.  Returns (sorted_ids, expert_ids,

@@ -3,8 +3,8 @@
 from . import workloads
 from .awq import AWQConfig, AWQLinearMethod, AWQMoEMethod
 from .ops import (awq_dequantize, awq_gemm, fused_moe_awq, moe_align_block_size, moe_awq_gemm,
-                  moe_sum, silu_and_mul, topk_softmax)
+                  moe_sum, silu_and_mul, topk_route, topk_softmax)
 
 __all__ = ["AWQConfig", "AWQLinearMethod", "AWQMoEMethod", "awq_dequantize", "awq_gemm",
            "fused_moe_awq", "moe_align_block_size", "moe_awq_gemm", "moe_sum", "silu_and_mul",
-           "topk_softmax", "workloads"]
+           "topk_route", "topk_softmax", "workloads"]

@@ -21,6 +21,8 @@ SIGNATURES = {
     "awqmi_gemm_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "awqmi_moe_topk_softmax_f32": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "awqmi_moe_topk_f32": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, ctypes.c_float, c_void_p,
+                                   c_void_p, c_void_p]),
     "awqmi_moe_align_capacity": (c_size_t, [c_int, c_int, c_int]),
     "awqmi_moe_align": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "awqmi_moe_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),

@@ -185,16 +185,19 @@ class AWQMoEMethod:
               renormalize: bool = True, use_grouped_topk: bool = False, topk_group: Optional[int] = None,
               num_expert_group: Optional[int] = None, global_num_experts: int = -1, expert_map=None,
               custom_routing_function=None, scoring_func: str = "softmax", e_score_correction_bias=None,
-              activation: str = "silu", **unused) -> torch.Tensor:
-        """Same keyword surface as vLLM's fused-MoE methods.  Supported: softmax scoring, plain
-        top-k (optionally renormalised), SiLU, all experts local; anything else is refused
+              activation: str = "silu", routed_scaling_factor: float = 1.0, **unused) -> torch.Tensor:
+        """Same keyword surface as vLLM's fused-MoE methods.  Supported: softmax or sigmoid
+        scoring, a score-correction bias (sigmoid), top-k over one expert group (optionally
+        renormalised, optionally scaled), SiLU, all experts local; anything else is refused
         rather than silently computed differently."""
-        if use_grouped_topk or topk_group or num_expert_group:
-            raise NotImplementedError("grouped top-k routing is not implemented")
-        if custom_routing_function is not None or e_score_correction_bias is not None:
-            raise NotImplementedError("custom routing / score correction bias is not implemented")
-        if scoring_func != "softmax":
-            raise NotImplementedError(f"scoring function {scoring_func!r} is not implemented (softmax only)")
+        if (topk_group or 1) > 1 or (num_expert_group or 1) > 1:
+            raise NotImplementedError("top-k over more than one expert group is not implemented")
+        if custom_routing_function is not None:
+            raise NotImplementedError("custom routing functions are not implemented")
+        if scoring_func not in ("softmax", "sigmoid"):
+            raise NotImplementedError(f"scoring function {scoring_func!r} is not implemented")
+        if e_score_correction_bias is not None and scoring_func != "sigmoid":
+            raise NotImplementedError("a score-correction bias is only implemented for sigmoid scoring")
         if activation != "silu":
             raise NotImplementedError(f"activation {activation!r} is not implemented (silu only)")
         if expert_map is not None or (global_num_experts not in (-1, layer.w13_qweight.shape[0])):
@@ -203,5 +206,9 @@ class AWQMoEMethod:
         x2 = x.reshape(-1, shape[-1]).contiguous()
         out = ops.fused_moe_awq(x2, (layer.w13_qweight, layer.w13_scales, layer.w13_qzeros),
                                 (layer.w2_qweight, layer.w2_scales, layer.w2_qzeros),
-                                router_logits.reshape(-1, router_logits.shape[-1]), top_k, renormalize)
+                                router_logits.reshape(-1, router_logits.shape[-1]), top_k, renormalize,
+                                scoring_func=scoring_func,
+                                e_score_correction_bias=(None if e_score_correction_bias is None
+                                                         else e_score_correction_bias.float().contiguous()),
+                                routed_scaling_factor=routed_scaling_factor)
         return out.reshape(shape)

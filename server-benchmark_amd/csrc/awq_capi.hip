@@ -339,16 +339,24 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   return launch_status();
 }
 
-int awqmi_moe_topk_softmax_f32(const float* logits, int T, int E, int topk, int renormalize,
-                               int32_t* topk_ids, float* topk_weights, void* stream) {
+int awqmi_moe_topk_f32(const float* logits, const float* score_bias, int T, int E, int topk, int scoring,
+                       int renormalize, float scale, int32_t* topk_ids, float* topk_weights, void* stream) {
   if (!logits || !topk_ids || !topk_weights) return AWQMI_NULL_POINTER;
   if (T <= 0 || E <= 0) return AWQMI_BAD_SHAPE;
-  if (E > AWQMI_MAX_EXPERTS || topk <= 0 || topk > E || topk > 64) return AWQMI_BAD_ARGUMENT;
+  if (E > AWQMI_MAX_EXPERTS || topk <= 0 || topk > E || topk > 64 || (scoring != 0 && scoring != 1))
+    return AWQMI_BAD_ARGUMENT;
+  if (scoring == 0 && score_bias) return AWQMI_BAD_ARGUMENT;   // the bias belongs to sigmoid scoring
   const dim3 grid((T + 3) / 4);
   hipStream_t st = (hipStream_t)stream;
-#define AWQMI_TOPK(P) \
-  hipLaunchKernelGGL(moe_topk_softmax_kernel<P>, grid, dim3(256), 0, st, logits, T, E, topk, renormalize, \
-                     topk_ids, topk_weights)
+#define AWQMI_TOPK(P)                                                                              \
+  do {                                                                                             \
+    if (scoring == 1)                                                                              \
+      hipLaunchKernelGGL((moe_topk_kernel<P, true>), grid, dim3(256), 0, st, logits, score_bias, T, E, topk, \
+                         renormalize, scale, topk_ids, topk_weights);                              \
+    else                                                                                           \
+      hipLaunchKernelGGL((moe_topk_kernel<P, false>), grid, dim3(256), 0, st, logits, score_bias, T, E, topk, \
+                         renormalize, scale, topk_ids, topk_weights);                              \
+  } while (0)
   if (E <= 64) AWQMI_TOPK(1);
   else if (E <= 128) AWQMI_TOPK(2);
   else if (E <= 256) AWQMI_TOPK(4);
@@ -356,6 +364,11 @@ int awqmi_moe_topk_softmax_f32(const float* logits, int T, int E, int topk, int 
   else AWQMI_TOPK(16);
 #undef AWQMI_TOPK
   return launch_status();
+}
+
+int awqmi_moe_topk_softmax_f32(const float* logits, int T, int E, int topk, int renormalize,
+                               int32_t* topk_ids, float* topk_weights, void* stream) {
+  return awqmi_moe_topk_f32(logits, nullptr, T, E, topk, 0, renormalize, 1.f, topk_ids, topk_weights, stream);
 }
 
 size_t awqmi_moe_align_capacity(int n_slots, int E, int tile_m) {

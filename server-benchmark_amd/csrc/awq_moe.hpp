@@ -7,53 +7,68 @@
 
 namespace awqmi {
 
-// One wave per token.  Selection runs on the raw logits (softmax is monotonic), ties go to
-// the lowest expert id.  PER = experts per lane (E <= 64 * PER).
-template <int PER>
-__global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __restrict__ logits, int T,
-                                                               int E, int topk, int renorm,
-                                                               int* __restrict__ ids,
-                                                               float* __restrict__ wts) {
+// One wave per token.  PER = experts per lane (E <= 64 * PER).
+// SIGMOID = false: softmax scores; selection runs on the raw logits (softmax is monotonic).
+// SIGMOID = true: score = sigmoid(logit); selection runs on score + bias[e] (bias may be
+// null), the weight is the score itself.  Ties go to the lowest expert id.  Weights are
+// optionally renormalised over the selected experts and multiplied by `scale`.
+template <int PER, bool SIGMOID>
+__global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__ logits,
+                                                       const float* __restrict__ bias, int T, int E,
+                                                       int topk, int renorm, float scale,
+                                                       int* __restrict__ ids, float* __restrict__ wts) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
-  float v[PER];
+  float v[PER];      // selection key
+  float sc[PER];     // score (SIGMOID only)
   float mx = -INFINITY;
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int e = lane + 64 * i;
-    v[i] = e < E ? logits[(size_t)t * E + e] : -INFINITY;
-    mx = fmaxf(mx, v[i]);
+    const float x = e < E ? logits[(size_t)t * E + e] : -INFINITY;
+    if (SIGMOID) {
+      sc[i] = 1.f / (1.f + __expf(-x));
+      v[i] = e < E ? sc[i] + (bias ? bias[e] : 0.f) : -INFINITY;
+    } else {
+      sc[i] = 0.f;
+      v[i] = x;
+      mx = fmaxf(mx, x);
+    }
   }
+  float sum = 1.f;
+  if (!SIGMOID) {
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-  float sum = 0.f;
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    sum = 0.f;
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    const int e = lane + 64 * i;
-    if (e < E) sum += __expf(v[i] - mx);
+    for (int i = 0; i < PER; ++i) {
+      const int e = lane + 64 * i;
+      if (e < E) sum += __expf(v[i] - mx);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
   }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
 
   float sel_sum = 0.f;
   float my_w = 0.f;   // lane j keeps the weight of pick j (topk <= 64)
   int my_id = 0;
   for (int it = 0; it < topk; ++it) {
-    float best = -INFINITY;
+    float best = -INFINITY, bsc = 0.f;
     int bidx = 0x7fffffff;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int e = lane + 64 * i;
-      if (e < E && (v[i] > best)) { best = v[i]; bidx = e; }   // ascending e: first max wins
+      if (e < E && (v[i] > best)) { best = v[i]; bidx = e; bsc = sc[i]; }   // ascending e: first max wins
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
       const float ob = __shfl_xor(best, o);
       const int oi = __shfl_xor(bidx, o);
-      if (ob > best || (ob == best && oi < bidx)) { best = ob; bidx = oi; }
+      const float os = SIGMOID ? __shfl_xor(bsc, o) : 0.f;
+      if (ob > best || (ob == best && oi < bidx)) { best = ob; bidx = oi; bsc = os; }
     }
-    const float pw = __expf(best - mx) / sum;
+    const float pw = SIGMOID ? bsc : __expf(best - mx) / sum;
     sel_sum += pw;
     if (lane == it) { my_w = pw; my_id = bidx; }
 #pragma unroll
@@ -62,7 +77,7 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __re
   }
   if (lane < topk) {
     ids[(size_t)t * topk + lane] = my_id;
-    wts[(size_t)t * topk + lane] = renorm ? my_w / sel_sum : my_w;
+    wts[(size_t)t * topk + lane] = (renorm ? my_w / sel_sum : my_w) * scale;
   }
 }
 

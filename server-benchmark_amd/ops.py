@@ -128,6 +128,35 @@ def topk_softmax(gating_output: torch.Tensor, topk: int, renormalize: bool = Tru
     return wts, ids
 
 
+def topk_route(gating_output: torch.Tensor, topk: int, renormalize: bool = True, scoring_func: str = "softmax",
+               e_score_correction_bias: torch.Tensor | None = None, routed_scaling_factor: float = 1.0):
+    """Routing with the scoring variants vLLM's fused MoE knows: "softmax" (plain top-k of the
+    softmax) or "sigmoid" (experts chosen by sigmoid(logit) + e_score_correction_bias, weighted
+    by sigmoid(logit)); weights optionally renormalised, then scaled.  Returns (weights, ids)."""
+    _need(gating_output, "gating_output", torch.float32, 2)
+    if scoring_func not in ("softmax", "sigmoid"):
+        raise ValueError(f"scoring_func must be 'softmax' or 'sigmoid', got {scoring_func!r}")
+    T, E = gating_output.shape
+    bias_ptr = 0
+    if e_score_correction_bias is not None:
+        if scoring_func != "sigmoid":
+            raise ValueError("e_score_correction_bias goes with sigmoid scoring")
+        _need(e_score_correction_bias, "e_score_correction_bias", torch.float32, 1)
+        if e_score_correction_bias.shape[0] != E:
+            raise ValueError(f"e_score_correction_bias has {e_score_correction_bias.shape[0]} entries, expected {E}")
+        bias_ptr = e_score_correction_bias.data_ptr()
+    ids = torch.empty((T, topk), dtype=torch.int32, device=gating_output.device)
+    wts = torch.empty((T, topk), dtype=torch.float32, device=gating_output.device)
+    if T == 0:
+        return wts, ids
+    st = _lib.load().awqmi_moe_topk_f32(gating_output.data_ptr(), bias_ptr, T, E, topk,
+                                        1 if scoring_func == "sigmoid" else 0, int(renormalize),
+                                        float(routed_scaling_factor), ids.data_ptr(), wts.data_ptr(),
+                                        _stream_ptr(gating_output.device))
+    _lib.check(st, "topk_route")
+    return wts, ids
+
+
 def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int):
     """Returns (sorted_token_ids, expert_ids, num_tokens_post_padded): flat slot indices
     stably sorted by expert, each expert's run padded to a multiple of block_size with the
@@ -214,15 +243,20 @@ def moe_sum(x: torch.Tensor, T: int, topk: int) -> torch.Tensor:
 
 
 def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Tensor, topk: int,
-                  renormalize: bool = True, block_size: int | None = None) -> torch.Tensor:
+                  renormalize: bool = True, block_size: int | None = None, scoring_func: str = "softmax",
+                  e_score_correction_bias: torch.Tensor | None = None,
+                  routed_scaling_factor: float = 1.0) -> torch.Tensor:
     """One AWQ MoE block: route -> align -> grouped GEMM (w13) -> SiLU*up -> grouped GEMM (w2,
     scaled by the routing weight) -> sum over slots.  w13 / w2 are (qweight, scales, qzeros)
     with a leading expert dimension; w13 columns are [gate | up].  With block_size left at
-    None the block runs as one library call; a block size selects the step-by-step path."""
+    None and plain softmax routing the block runs as one library call; a block size, sigmoid
+    scoring, a score-correction bias or a routed scaling factor select the step-by-step path."""
     _need(hidden_states, "hidden_states", torch.float16, 2)
     T, H = hidden_states.shape
     E = w13[0].shape[0]
-    if block_size is None:
+    plain_routing = (scoring_func == "softmax" and e_score_correction_bias is None
+                     and routed_scaling_factor == 1.0)
+    if block_size is None and plain_routing:
         # the whole block in one library call, intermediates in the workspace
         for i, (t, dt) in enumerate(zip(tuple(w13) + tuple(w2), (torch.int32, torch.float16, torch.int32) * 2)):
             _need(t, f"w13/w2[{i}]", dt, 3)
@@ -249,7 +283,8 @@ def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Ten
         return out
     T = hidden_states.shape[0]
     E = w13[0].shape[0]
-    topk_w, topk_ids = topk_softmax(gating_output.float().contiguous(), topk, renormalize)
+    topk_w, topk_ids = topk_route(gating_output.float().contiguous(), topk, renormalize, scoring_func,
+                                  e_score_correction_bias, routed_scaling_factor)
     n = T * topk
     # 16-row blocks measured faster than 32-row blocks at every token count tried (the
     # two-row-block instantiation of the skinny kernel is issue-bound)

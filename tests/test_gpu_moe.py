@@ -210,3 +210,29 @@ def test_fused_activation_agrees_with_step_by_step(sba, gpu, T):
     ref = _dense_expert_reference(sba, c, gpu, T, 2048, 128, 8, 768)
     assert float((one.float() - ref).norm() / ref.norm()) <= TOL
     assert torch.equal(one, sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 8, True))
+
+
+@pytest.mark.parametrize("T,E,topk", [(1, 128, 8), (33, 128, 8), (7, 160, 6), (5, 16, 2)])
+def test_topk_sigmoid_with_bias(sba, gpu, T, E, topk):
+    g = torch.Generator().manual_seed(T * 3 + E)
+    logits = torch.randn((T, E), generator=g)
+    bias = torch.randn((E,), generator=g) * 0.1
+    for renorm, b, scale in ((True, bias, 2.5), (False, None, 1.0), (True, None, 1.0)):
+        w, ids = sba.topk_route(logits.to(gpu), topk, renorm, "sigmoid", None if b is None else b.to(gpu), scale)
+        rid, rw = awq_ref.topk_sigmoid(logits.numpy(), topk, renorm, None if b is None else b.numpy(), scale)
+        assert np.array_equal(ids.cpu().numpy(), rid)
+        assert np.allclose(w.cpu().numpy(), rw, rtol=2e-5, atol=1e-8)
+
+
+def test_moe_block_sigmoid_routing(sba, gpu):
+    """The block with sigmoid routing + bias + scaling factor against the oracle's forward with
+    the oracle's routing."""
+    c = sba.workloads.make_moe_case(12, 256, 16, 4, 128, 128, seed=77)
+    bias = (torch.randn((16,), generator=torch.Generator().manual_seed(5)) * 0.1)
+    cg = c.to(gpu)
+    y = sba.fused_moe_awq(cg.x, cg.w13, cg.w2, cg.logits, 4, True, scoring_func="sigmoid",
+                          e_score_correction_bias=bias.to(gpu), routed_scaling_factor=1.5).cpu().numpy()
+    ids, tw = awq_ref.topk_sigmoid(c.logits.numpy(), 4, True, bias.numpy(), 1.5)
+    ref = awq_ref.moe_forward(c.x.numpy(), tuple(a.numpy() for a in c.w13), tuple(a.numpy() for a in c.w2),
+                              ids, tw, 128)
+    assert awq_ref.rel_frobenius(y, ref) <= TOL

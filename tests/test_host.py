@@ -198,7 +198,8 @@ def test_moe_method_refuses_unsupported_routing(sba):
     layer = torch.nn.Module()
     m.create_weights(layer, 4, 256, 128, torch.float16)
     x, lg = torch.zeros((2, 256), dtype=torch.float16), torch.zeros((2, 4))
-    for kw in (dict(use_grouped_topk=True), dict(scoring_func="sigmoid"), dict(activation="gelu"),
+    for kw in (dict(use_grouped_topk=True, num_expert_group=4, topk_group=2), dict(scoring_func="tanh"),
+               dict(activation="gelu"), dict(e_score_correction_bias=torch.zeros(4)),
                dict(expert_map=torch.arange(4)), dict(global_num_experts=8),
                dict(custom_routing_function=lambda *a: None)):
         with pytest.raises(NotImplementedError):

@@ -315,3 +315,23 @@ def test_moe_forward_against_grouped_formulation():
             a = h[:I] / (1 + np.exp(-h[:I])) * h[I:]
             want[t] += (a @ W2) * tw[t, slot]
     assert awq_ref.rel_frobenius(got, want) < 2e-3
+
+
+def test_topk_sigmoid_matches_torch():
+    import torch
+    """sigmoid scoring with a correction bias: ids from torch.topk of score + bias, weights the
+    plain scores (random floats: no ties), renormalised and scaled."""
+    g = torch.Generator().manual_seed(11)
+    logits = torch.randn((9, 40), generator=g)
+    bias = torch.randn((40,), generator=g) * 0.1
+    score = torch.sigmoid(logits.double())
+    choice = score.float() + bias
+    ids_t = torch.topk(choice, 5, dim=-1).indices
+    w_t = score.gather(1, ids_t)
+    w_t = w_t / w_t.sum(dim=-1, keepdim=True) * 2.5
+    ids, w = awq_ref.topk_sigmoid(logits.numpy(), 5, True, bias.numpy(), 2.5)
+    assert np.array_equal(ids, ids_t.numpy().astype(np.int32))
+    assert np.allclose(w, w_t.numpy(), rtol=1e-6)
+    ids2, w2 = awq_ref.topk_sigmoid(logits.numpy(), 5, False)
+    assert np.array_equal(ids2, torch.topk(score, 5, dim=-1).indices.numpy().astype(np.int32))
+    assert np.allclose(w2, torch.topk(score, 5, dim=-1).values.numpy(), rtol=1e-6)
