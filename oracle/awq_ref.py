@@ -24,10 +24,11 @@ Parity status per function (what pins it, independent of this file's own formula
   gemm                    library fp64 matmul on pinned W, one-hot / w==z cases  PINNED
   moe_align               permutation / padding invariants                       PINNED
   topk_softmax            torch.softmax + torch.topk                             PINNED
+  topk_sigmoid            torch.sigmoid + torch.topk of score + bias             PINNED
   moe_forward             per-token brute force from pinned W                    PINNED
   behavioural choices only an import of vLLM could pin (M threshold between fused GEMM
   and dequant+matmul, sentinel/padding layout of its align kernel, [gate | up] order
-  inside w13)                                                         PARITY UNPINNED
+  inside w13, where its grouped top-k applies the scaling factor)     PARITY UNPINNED
 """
 from __future__ import annotations
 
