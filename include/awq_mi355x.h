@@ -114,9 +114,10 @@ int awqmi_moe_align(const int32_t* topk_ids, int n_slots, int E, int tile_m,
 /* Workspace bytes of one grouped GEMM call (same counter rule as awqmi_gemm_f16). */
 size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int split_k, int tile_m);
 
-/* Expert-grouped AWQ GEMM over sorted-token blocks of tile_m rows (16, or 32 when the
- * average expert load makes 16-row blocks re-read weights; the ids must come from
- * awqmi_moe_align with the same tile_m).
+/* Expert-grouped AWQ GEMM over sorted-token blocks of tile_m rows; the ids must come from
+ * awqmi_moe_align with the same tile_m.  tile_m 16 or 32: the skinny kernel (decode-sized
+ * batches).  tile_m 64, 128 or 256: the MFMA kernel, for many slots per expert; it takes no
+ * split_k or workspace and needs x and each expert's tensors under 4 GiB.
  * For every non-pad entry s = sorted_token_ids[i] in a block owned by expert e:
  *     y[s, :] = (x[s / a_row_div, :] @ W_e) * (topk_weights ? topk_weights[s] : 1)
  * a_row_div = topk for the first GEMM (x is [T, K]), 1 for the second (x is [n_slots, K]).

@@ -432,7 +432,10 @@ static MoePlan moe_plan(int n_slots, int E, int K, int N, int tile_m, int split_
 }
 
 size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int split_k, int tile_m) {
-  if (n_slots <= 0 || E <= 0 || K <= 0 || N <= 0 || N % 8 != 0 || (tile_m != 16 && tile_m != 32)) return 0;
+  if (n_slots <= 0 || E <= 0 || K <= 0 || N <= 0 || N % 8 != 0 ||
+      (tile_m != 16 && tile_m != 32 && tile_m != 64 && tile_m != 128 && tile_m != 256))
+    return 0;
+  if (tile_m >= 64) return AWQMI_WS_COUNTER_BYTES;    // the grouped MFMA form needs no partials
   const MoePlan pl = moe_plan(n_slots, E, K, N, tile_m, split_k);
   return AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, pl.split, pl.nblk, tile_m);
 }
@@ -476,13 +479,64 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   if (int st = check_awq_shape(K, N, G)) return st;
   if (n_slots <= 0 || E <= 0) return AWQMI_BAD_SHAPE;
   if (a_row_div <= 0 || split_k < 0 || split_k > AWQMI_MAX_SPLIT_K || E > AWQMI_MAX_EXPERTS ||
-      (tile_m != 16 && tile_m != 32))
+      (tile_m != 16 && tile_m != 32 && tile_m != 64 && tile_m != 128 && tile_m != 256))
     return AWQMI_BAD_ARGUMENT;
   if (!gemv_tiled_ok(K, G)) return AWQMI_UNSUPPORTED_GROUP;
   if (!aligned16(x) || !aligned16(scales) || !aligned16(qweight) || !aligned16(qzeros) ||
       !aligned16(y))
     return AWQMI_BAD_ALIGN;
   const int NW = N / 8;
+  if (tile_m >= 64) {
+    // blocks of 64 / 128 slots: the MFMA kernel in its expert-grouped form (no K split)
+    if (fuse_act) return AWQMI_BAD_ARGUMENT;
+    const size_t x_rows = ((size_t)n_slots + a_row_div - 1) / a_row_div;
+    if (x_rows * K * 2 >= (1ull << 32) || (size_t)K * NW * 4 >= (1ull << 32) ||
+        (size_t)(K / G) * N * 2 >= (1ull << 32))
+      return AWQMI_BAD_SHAPE;
+    static std::atomic<bool> gattr{false};
+    if (!gattr.load(std::memory_order_acquire)) {
+      const void* fns[6] = {reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1, 8, true>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1, 8, true>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 2, 8, true>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 2, 8, true>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4, 4, true>),
+                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 4, 4, true>)};
+      for (const void* fn : fns) {
+        const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, PF_LDS_BYTES);
+        if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
+      }
+      gattr.store(true, std::memory_order_release);
+    }
+    MfmaGemmParams p{};
+    p.x = reinterpret_cast<const half_t*>(x);
+    p.qw = reinterpret_cast<const uint32_t*>(qweight);
+    p.sc = reinterpret_cast<const half_t*>(scales);
+    p.qz = reinterpret_cast<const uint32_t*>(qzeros);
+    p.y = reinterpret_cast<half_t*>(y);
+    p.M = (int)x_rows; p.K = K; p.N = N; p.NW = NW; p.G = G;
+    const bool pow2g = (G & (G - 1)) == 0 && G >= 8;
+    p.gshift = 0;
+    if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
+    p.mt = 1; p.nt = (N + PF_BN - 1) / PF_BN; p.total = p.nt; p.per_xcd = 0;
+    p.dp_tiles = 0; p.sk_tiles = 0; p.sk_split = 1;
+    p.sorted_ids = sorted_token_ids; p.expert_ids = expert_ids; p.n_post_pad = num_tokens_post_padded;
+    p.topk_w = topk_weights; p.n_slots = n_slots; p.a_row_div = a_row_div;
+    p.w_stride = (long long)K * NW; p.s_stride = (long long)(K / G) * N; p.z_stride = (long long)(K / G) * NW;
+    const int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, tile_m) / tile_m);
+    const dim3 grid((unsigned)nblk * p.nt);
+    hipStream_t st = (hipStream_t)stream;
+    if (tile_m == 64) {
+      if (pow2g) hipLaunchKernelGGL((awq_gemm_mfma_kernel<true, 1, 8, true>), grid, dim3(512), PF_LDS_BYTES, st, p);
+      else hipLaunchKernelGGL((awq_gemm_mfma_kernel<false, 1, 8, true>), grid, dim3(512), PF_LDS_BYTES, st, p);
+    } else if (tile_m == 128) {
+      if (pow2g) hipLaunchKernelGGL((awq_gemm_mfma_kernel<true, 2, 8, true>), grid, dim3(512), PF_LDS_BYTES, st, p);
+      else hipLaunchKernelGGL((awq_gemm_mfma_kernel<false, 2, 8, true>), grid, dim3(512), PF_LDS_BYTES, st, p);
+    } else {
+      if (pow2g) hipLaunchKernelGGL((awq_gemm_mfma_kernel<true, 4, 4, true>), grid, dim3(256), PF_LDS_BYTES, st, p);
+      else hipLaunchKernelGGL((awq_gemm_mfma_kernel<false, 4, 4, true>), grid, dim3(256), PF_LDS_BYTES, st, p);
+    }
+    return launch_status();
+  }
   const MoePlan pl = moe_plan(n_slots, E, K, N, tile_m, split_k);
   const int wpl = pl.wpl, ncb = pl.ncb, nblk = pl.nblk, split = pl.split;
   if (tile_m == 32 && wpl != 2) return AWQMI_BAD_SHAPE;   // 32-row blocks need N % 16 == 0
@@ -559,26 +613,64 @@ int awqmi_moe_sum_f16(const void* in, void* out, int T, int topk, int H, void* s
 }
 
 namespace {
+// Rows per block for the two expert GEMMs of one MoE block: 16 (the skinny kernel) or 64 /
+// 128 / 256 (the MFMA kernel's expert-grouped form).  Cost model fitted on measurements over
+// three expert shapes (2048/768 x 128 experts, 6144/2560 x 160, 4096/14336 x 8):
+//   skinny: flops / (440 TFLOP/s * avg / (avg + 24)), avg = slots per expert;
+//   MFMA:   per GEMM blocks * column tiles / 256 CUs rounds (a partial last round counts as
+//           at least half) of (K / 64 + overhead) k-tiles at 5.7 ns * (rows + 96) each, plus
+//           the separate SiLU pass at 4 TB/s; blocks is the expected block count after
+//           padding each expert's run to whole blocks.
+// Within about 15 % of the best choice on every measured point.
+// The MFMA form also needs every operand under 4 GiB (32-bit buffer offsets).
+int moe_pick_tile(int n_slots, int E, int H, int inter, int group) {
+  const int v = g_gemv_variant.load(std::memory_order_relaxed);
+  if (v >= 0 && (v & 2048)) return 16;
+  if (!gemv_tiled_ok(H, norm_group(H, group)) || !gemv_tiled_ok(inter, norm_group(inter, group))) return 16;
+  if ((size_t)n_slots * std::max(H, inter) * 2 >= (1ull << 32) ||
+      (size_t)H * (2 * inter / 8) * 4 >= (1ull << 32) || (size_t)inter * (H / 8) * 4 >= (1ull << 32))
+    return 16;
+  const double avg = (double)n_slots / E;
+  const double flops = 2.0 * n_slots * ((double)H * 2 * inter + (double)inter * H);
+  double best = flops / (440e12 * avg / (avg + 24.0));
+  int tile = 16;
+  for (int bm : {64, 128, 256}) {
+    const double blocks = avg >= bm ? (double)n_slots / bm + 0.5 * E : E * (1.0 + avg / (4.0 * bm));
+    const double kt_s = 5.7e-9 * (bm + 96);
+    const int over = bm == 256 ? 10 : 6;
+    auto gemm = [&](int K, int N) {
+      const double r = blocks * ((N + PF_BN - 1) / PF_BN) / 256.0;
+      const double whole = std::floor(r), part = r - whole;
+      const double rounds = whole + (part > 0 ? std::max(part, 0.5) : 0.0);
+      return rounds * (K / PF_BK + over) * kt_s;
+    };
+    const double t = gemm(H, 2 * inter) + gemm(inter, H) + 5e-6 + 6.0 * n_slots * inter / 4e12;
+    if (t < best) { best = t; tile = bm; }
+  }
+  return tile;
+}
+
 // workspace carve-up of the fused MoE block; every piece starts 256-byte aligned
 struct FusedMoeLayout {
   size_t gemm_ws, ids, wts, sorted, experts, npp, h13, act, o, total;
   size_t gemm_ws_bytes;
-  int n_slots, cap;
+  int n_slots, cap, tile;
 };
-FusedMoeLayout fused_moe_layout(int T, int H, int inter, int E, int topk) {
+FusedMoeLayout fused_moe_layout(int T, int H, int inter, int E, int topk, int tile) {
   FusedMoeLayout L{};
   auto up = [](size_t v) { return (v + 255) / 256 * 256; };
   L.n_slots = T * topk;
-  L.cap = (int)awqmi_moe_align_capacity(L.n_slots, E, 16);
-  const size_t g1 = awqmi_moe_gemm_workspace_bytes(L.n_slots, E, H, 2 * inter, 0, 16);
-  const size_t g2 = awqmi_moe_gemm_workspace_bytes(L.n_slots, E, inter, H, 0, 16);
+  L.tile = tile;
+  L.cap = (int)awqmi_moe_align_capacity(L.n_slots, E, L.tile);
+  const size_t g1 = awqmi_moe_gemm_workspace_bytes(L.n_slots, E, H, 2 * inter, 0, L.tile);
+  const size_t g2 = awqmi_moe_gemm_workspace_bytes(L.n_slots, E, inter, H, 0, L.tile);
   L.gemm_ws_bytes = g1 > g2 ? g1 : g2;
   size_t off = 0;
   L.gemm_ws = off; off += up(L.gemm_ws_bytes);
   L.ids = off;     off += up((size_t)L.n_slots * 4);
   L.wts = off;     off += up((size_t)L.n_slots * 4);
   L.sorted = off;  off += up((size_t)L.cap * 4);
-  L.experts = off; off += up((size_t)(L.cap / 16) * 4);
+  L.experts = off; off += up((size_t)(L.cap / L.tile) * 4);
   L.npp = off;     off += 256;
   L.h13 = off;     off += up((size_t)L.n_slots * 2 * inter * 2);
   L.act = off;     off += up((size_t)L.n_slots * inter * 2);
@@ -591,7 +683,9 @@ FusedMoeLayout fused_moe_layout(int T, int H, int inter, int E, int topk) {
 size_t awqmi_fused_moe_workspace_bytes(int T, int H, int inter, int E, int topk) {
   if (T <= 0 || H <= 0 || inter <= 0 || E <= 0 || topk <= 0 || H % 8 != 0 || inter % 8 != 0) return 0;
   if ((long long)T * topk > (1LL << 30)) return 0;
-  return fused_moe_layout(T, H, inter, E, topk).total;
+  size_t most = 0;     // the call picks the block rows from the shapes; any choice fits
+  for (int tile : {16, 64, 128, 256}) most = std::max(most, fused_moe_layout(T, H, inter, E, topk, tile).total);
+  return most;
 }
 
 int awqmi_fused_moe_f16(const void* hidden, const float* router_logits, const int32_t* w13_q,
@@ -606,7 +700,8 @@ int awqmi_fused_moe_f16(const void* hidden, const float* router_logits, const in
   if (topk <= 0 || topk > E || topk > 64 || E > AWQMI_MAX_EXPERTS || (long long)T * topk > (1LL << 30))
     return AWQMI_BAD_ARGUMENT;
   if (!aligned16(workspace)) return AWQMI_BAD_ALIGN;
-  const FusedMoeLayout L = fused_moe_layout(T, H, inter, E, topk);
+  const int tile = moe_pick_tile(T * topk, E, H, inter, group);
+  const FusedMoeLayout L = fused_moe_layout(T, H, inter, E, topk, tile);
   if (workspace_bytes < L.total) return AWQMI_WORKSPACE_TOO_SMALL;
   char* ws = static_cast<char*>(workspace);
   int32_t* ids = reinterpret_cast<int32_t*>(ws + L.ids);
@@ -619,10 +714,10 @@ int awqmi_fused_moe_f16(const void* hidden, const float* router_logits, const in
   void* o = ws + L.o;
   int st = awqmi_moe_topk_softmax_f32(router_logits, T, E, topk, renormalize, ids, wts, stream);
   if (st) return st;
-  st = awqmi_moe_align(ids, L.n_slots, E, 16, sorted, experts, npp, stream);
+  st = awqmi_moe_align(ids, L.n_slots, E, tile, sorted, experts, npp, stream);
   if (st) return st;
   const int Gn = norm_group(H, group);
-  if (gemv_tiled_ok(H, Gn) && moe_can_fuse_act(L.n_slots, E, H, 2 * inter) &&
+  if (tile == 16 && gemv_tiled_ok(H, Gn) && moe_can_fuse_act(L.n_slots, E, H, 2 * inter) &&
       !(g_gemv_variant.load(std::memory_order_relaxed) >= 0 &&
         (g_gemv_variant.load(std::memory_order_relaxed) & 1024))) {
     // the w13 GEMM writes silu(gate) * up itself
@@ -631,12 +726,12 @@ int awqmi_fused_moe_f16(const void* hidden, const float* router_logits, const in
     if (st) return st;
   } else {
     st = awqmi_moe_gemm_f16(hidden, w13_q, w13_s, w13_z, h13, sorted, experts, npp, nullptr, L.n_slots, topk,
-                            16, E, H, 2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream);
+                            tile, E, H, 2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream);
     if (st) return st;
     st = awqmi_silu_and_mul_f16(h13, act, L.n_slots, inter, stream);
     if (st) return st;
   }
-  st = awqmi_moe_gemm_f16(act, w2_q, w2_s, w2_z, o, sorted, experts, npp, wts, L.n_slots, 1, 16, E, inter, H,
+  st = awqmi_moe_gemm_f16(act, w2_q, w2_s, w2_z, o, sorted, experts, npp, wts, L.n_slots, 1, tile, E, inter, H,
                           group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream);
   if (st) return st;
   return awqmi_moe_sum_f16(o, out, T, topk, H, stream);

@@ -45,6 +45,15 @@ struct MfmaGemmParams {
   // tile would have to pull sk_split x 256 KiB by itself, which took longer than the GEMM).
   int dp_tiles, sk_tiles, sk_split;
   float* sk_part;   // [sk_tiles][sk_split][256 * 256] fp32
+  // Expert-grouped launch (kernel instantiation GROUPED): workgroup (blk, column tile); blk is
+  // a block of BM sorted slots of one expert (moe_align with tile_m = BM).
+  const int* sorted_ids;
+  const int* expert_ids;
+  const int* n_post_pad;
+  const float* topk_w;      // optional per-slot output weight
+  int n_slots;
+  int a_row_div;            // X row of a slot = slot / a_row_div
+  long long w_stride, s_stride, z_stride;   // elements per expert
 };
 
 constexpr int PF_SK_SLOT_FLOATS = 256 * 256;
@@ -78,7 +87,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* base, size
 // 8: two waves per SIMD, each 32 MI x 64, for MI <= 2: with half the accumulators two waves
 // fit, and the waits of one (fragment reads, the barrier, operand loads) are covered by the
 // MFMAs of the other -- the small tiles spend most of a k-tile in such waits otherwise.
-template <bool POW2G, int MI = 4, int NWV = 4>
+// GROUPED: the expert-grouped form for MoE batches with many rows per expert: X rows are
+// gathered through the sorted slot list, the weight triple is the block's expert's, output
+// rows go to their slot rows (times the routing weight when given).
+template <bool POW2G, int MI = 4, int NWV = 4, bool GROUPED = false>
 __global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const MfmaGemmParams p) {
   constexpr int BM = 64 * MI;            // workgroup tile rows
   constexpr int NTH = 64 * NWV;          // threads
@@ -93,8 +105,29 @@ __global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int id = blockIdx.x;
   const int KT = p.K / PF_BK;
-  int nid, kb = 0, ke = KT, part = -1;
-  if (id < 8 * p.per_xcd) {
+  int nid = 0, kb = 0, ke = KT, part = -1;
+  __shared__ int s_sid[GROUPED ? 64 * MI : 1];
+  __shared__ float s_tw[GROUPED ? 64 * MI : 1];
+  const uint32_t* qw_base = p.qw;
+  const uint32_t* qz_base = p.qz;
+  const half_t* sc_base = p.sc;
+  int g_m0 = 0, g_n0 = 0;
+  if (GROUPED) {
+    const int blk = id / p.nt;
+    if (blk * BM >= *p.n_post_pad) return;
+    const int e = p.expert_ids[blk];
+    qw_base += (size_t)e * p.w_stride;
+    qz_base += (size_t)e * p.z_stride;
+    sc_base += (size_t)e * p.s_stride;
+    g_m0 = blk * BM;
+    g_n0 = (id % p.nt) * PF_BN;
+    for (int r = tid; r < BM; r += NTH) {
+      const int sid = p.sorted_ids[g_m0 + r];
+      s_sid[r] = sid;
+      s_tw[r] = (sid < p.n_slots && p.topk_w) ? p.topk_w[sid] : 1.f;
+    }
+    __syncthreads();
+  } else if (id < 8 * p.per_xcd) {
     nid = (id & 7) * p.per_xcd + (id >> 3);
     if (nid >= p.dp_tiles) return;
   } else {
@@ -109,13 +142,13 @@ __global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const 
   const int gm = min(p.mt - first_m, 8);
   const int mt_i = first_m + (nid % gsize) % gm;
   const int nt_i = (nid % gsize) / gm;
-  const int m0 = mt_i * BM, n0 = nt_i * PF_BN;
+  const int m0 = GROUPED ? g_m0 : mt_i * BM, n0 = GROUPED ? g_n0 : nt_i * PF_BN;
   const int wm = (wave / (NWV / 2)) * (32 * MI), wn = (wave % (NWV / 2)) * (32 * NJ);
 
   const __amdgpu_buffer_rsrc_t rx = pf_rsrc(p.x, (size_t)p.M * p.K * 2);
-  const __amdgpu_buffer_rsrc_t rw = pf_rsrc(p.qw, (size_t)p.K * p.NW * 4);
-  const __amdgpu_buffer_rsrc_t rz = pf_rsrc(p.qz, (size_t)(p.K / p.G) * p.NW * 4);
-  const __amdgpu_buffer_rsrc_t rs = pf_rsrc(p.sc, (size_t)(p.K / p.G) * p.N * 2);
+  const __amdgpu_buffer_rsrc_t rw = pf_rsrc(qw_base, (size_t)p.K * p.NW * 4);
+  const __amdgpu_buffer_rsrc_t rz = pf_rsrc(qz_base, (size_t)(p.K / p.G) * p.NW * 4);
+  const __amdgpu_buffer_rsrc_t rs = pf_rsrc(sc_base, (size_t)(p.K / p.G) * p.N * 2);
 
   // ---- global -> LDS roles -------------------------------------------------------------
   // X tile: thread (a_row + 32 i, a_seg) moves 16 bytes; rows past M re-read row M - 1 (their
@@ -126,7 +159,13 @@ __global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const 
 #pragma unroll
   for (int i = 0; i < AL; ++i) {
     const int r = a_row + ARP * i;
-    const int gr = min(m0 + r, p.M - 1);
+    int gr;
+    if (GROUPED) {
+      const int sid = s_sid[r];
+      gr = sid < p.n_slots ? sid / p.a_row_div : 0;     // pad rows read row 0, never stored
+    } else {
+      gr = min(m0 + r, p.M - 1);
+    }
     a_off[i] = (uint32_t)(((size_t)gr * p.K + 8 * a_seg) * 2);
     a_dst[i] = r * PF_ROW_BYTES + ((a_seg ^ pf_swz(r)) << 4);
   }
@@ -370,8 +409,14 @@ __global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const 
       if (col >= p.N) continue;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm + 32 * i + 8 * (r >> 2) + row_l + (r & 3);
-        if (row < p.M) p.y[(size_t)row * p.N + col] = (half_t)acc[i][j][r];
+        const int lrow = wm + 32 * i + 8 * (r >> 2) + row_l + (r & 3);
+        if (GROUPED) {
+          const int sid = s_sid[lrow];
+          if (sid < p.n_slots) p.y[(size_t)sid * p.N + col] = (half_t)(acc[i][j][r] * s_tw[lrow]);
+        } else {
+          const int row = m0 + lrow;
+          if (row < p.M) p.y[(size_t)row * p.N + col] = (half_t)acc[i][j][r];
+        }
       }
     }
 }

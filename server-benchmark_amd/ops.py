@@ -180,7 +180,8 @@ def moe_awq_gemm(a: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, q
                  num_tokens_post_padded: torch.Tensor, n_slots: int, a_row_div: int,
                  topk_weights: torch.Tensor | None = None, split_k: int = 0,
                  out: torch.Tensor | None = None, block_size: int = MOE_TILE_M) -> torch.Tensor:
-    """Expert-grouped AWQ GEMM over blocks of `block_size` (16 or 32) sorted slots:
+    """Expert-grouped AWQ GEMM over blocks of `block_size` sorted slots (16 or 32: the skinny
+    kernel; 64, 128 or 256: the MFMA kernel in its expert-grouped form, for many rows per expert):
     out[s] = a[s // a_row_div] @ W[expert(s)] (* topk_weights[s]).  The ids must come from
     moe_align_block_size with the same block size."""
     _need(a, "a", torch.float16, 2)
@@ -197,8 +198,8 @@ def moe_awq_gemm(a: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, q
     if a.shape[0] * a_row_div < n_slots:
         raise ValueError("a has too few rows for n_slots / a_row_div")
     lib = _lib.load()
-    if block_size not in (16, 32):
-        raise ValueError("block_size must be 16 or 32")
+    if block_size not in (16, 32, 64, 128, 256):
+        raise ValueError("block_size must be 16, 32, 64, 128 or 256")
     cap = lib.awqmi_moe_align_capacity(n_slots, E, block_size)
     if sorted_token_ids.numel() < cap or expert_ids.numel() < cap // block_size:
         raise ValueError("sorted_token_ids / expert_ids smaller than the align capacity")

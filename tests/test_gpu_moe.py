@@ -91,6 +91,66 @@ def test_moe_grouped_gemm_block_sizes(sba, gpu, bs):
     assert err <= TOL
 
 
+@pytest.mark.parametrize("bs,T,E,topk,K,N,G", [
+    (64, 300, 6, 2, 256, 264, 128),     # ragged last column tile, ragged last blocks
+    (128, 300, 6, 2, 256, 264, 128),
+    (256, 300, 6, 2, 256, 264, 128),
+    (64, 97, 5, 1, 384, 512, 64),       # top-1, group 64, K = 6 k-tiles
+    (128, 1, 4, 2, 128, 256, 32),       # a single token: every block is nearly all padding
+    (128, 700, 3, 3, 640, 1024, 128),   # several blocks per expert
+])
+def test_moe_grouped_gemm_mfma_blocks(sba, gpu, bs, T, E, topk, K, N, G):
+    """The grouped GEMM over 64 / 128 / 256-row blocks (the MFMA kernel's expert-grouped form)
+    against per-slot oracle products, with routing weights."""
+    rng = np.random.default_rng(bs + T + K)
+    w = rng.integers(0, 16, (E, K, N))
+    z = rng.integers(0, 16, (E, K // G, N))
+    s = (rng.random((E, K // G, N)) * 0.019 + 0.001).astype(np.float16)
+    qw, qz = awq_ref.pack_awq(w), awq_ref.pack_awq(z)
+    x = rng.normal(0, 1, (T, K)).astype(np.float16)
+    ids = np.stack([rng.choice(E, size=topk, replace=False) for _ in range(T)]).astype(np.int32)
+    tw = rng.random((T, topk)).astype(np.float32)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+    sid, eid, npp = sba.moe_align_block_size(t(ids), bs, E)
+    out = torch.full((T * topk, N), float("nan"), dtype=torch.float16, device=gpu)
+    y = sba.moe_awq_gemm(t(x), t(qw), t(s), t(qz), sid, eid, npp, T * topk, topk, topk_weights=t(tw),
+                         block_size=bs, out=out).cpu().numpy()
+    assert np.all(np.isfinite(y))            # every slot row written
+    ref = np.zeros((T * topk, N))
+    for e in range(E):
+        tok, slot = np.nonzero(ids == e)
+        if tok.size:
+            ref[tok * topk + slot] = awq_ref.gemm_wide(x[tok], qw[e], s[e], qz[e], G) * tw[tok, slot][:, None]
+    err = awq_ref.rel_frobenius(y, ref)
+    print(f"[moe grouped mfma bs={bs} T={T}] rel_fro={err:.2e}", flush=True)
+    assert err <= TOL
+    # same ids, no routing weight, one X row per slot (the second expert GEMM's addressing)
+    xs = rng.normal(0, 1, (T * topk, K)).astype(np.float16)
+    y2 = sba.moe_awq_gemm(t(xs), t(qw), t(s), t(qz), sid, eid, npp, T * topk, 1, block_size=bs).cpu().numpy()
+    ref2 = np.zeros((T * topk, N))
+    flat = ids.reshape(-1)
+    for e in range(E):
+        rows = np.nonzero(flat == e)[0]
+        if rows.size:
+            ref2[rows] = awq_ref.gemm_wide(xs[rows], qw[e], s[e], qz[e], G)
+    assert awq_ref.rel_frobenius(y2, ref2) <= TOL
+
+
+@pytest.mark.parametrize("T,H,E,topk,I", [(2048, 2048, 128, 8, 768), (1024, 1024, 8, 2, 2048)])
+def test_fused_call_on_prefill_batches(sba, gpu, T, H, E, topk, I):
+    """Batches with many slots per expert, where the one-call path takes the MFMA blocks:
+    against the dense expert path and against the step-by-step path over 16-row blocks."""
+    c = sba.workloads.make_moe_case(T, H, E, topk, I, 128, seed=T + I).to(gpu)
+    one = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True)
+    ref = _dense_expert_reference(sba, c, gpu, T, H, E, topk, I)
+    err = float((one.float() - ref).norm() / ref.norm())
+    step = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True, block_size=16)
+    d = float((one.float() - step.float()).norm() / step.float().norm())
+    print(f"[moe prefill T={T} E={E}] vs dense experts {err:.2e}, vs 16-row blocks {d:.2e}", flush=True)
+    assert err <= TOL and d <= TOL
+    assert torch.equal(one, sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True))
+
+
 @pytest.mark.parametrize("T", [1, 16])
 def test_moe_qwen3_shapes_vs_oracle(sba, gpu, T):
     c = sba.workloads.make_moe_case(T, 2048, 128, 8, 768, 128, seed=100 + T)
@@ -193,6 +253,8 @@ def test_moe_odd_shapes_vs_dense_expert_path(sba, gpu, T, H, E, topk, I):
     print(f"[moe odd T={T} E={E} topk={topk}] rel_fro={err:.2e}", flush=True)
     assert err <= TOL
     assert torch.equal(y, sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True))
+    y16 = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True, block_size=16)
+    assert float((y16.float() - ref).norm() / ref.norm()) <= TOL
 
 
 @pytest.mark.parametrize("T", [128, 512])

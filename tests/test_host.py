@@ -77,11 +77,13 @@ def test_fused_moe_workspace_covers_every_intermediate(lib):
     T, H, I, E, topk = 16, 2048, 768, 128, 8
     n = T * topk
     total = lib.awqmi_fused_moe_workspace_bytes(T, H, I, E, topk)
-    g = max(lib.awqmi_moe_gemm_workspace_bytes(n, E, H, 2 * I, 0, 16),
-            lib.awqmi_moe_gemm_workspace_bytes(n, E, I, H, 0, 16))
-    cap = lib.awqmi_moe_align_capacity(n, E, 16)
-    payload = g + 2 * n * 4 + cap * 4 + cap // 16 * 4 + 4 + n * 2 * I * 2 + n * I * 2 + n * H * 2
-    assert payload <= total <= payload + 9 * 256
+    payloads = []
+    for tile in (16, 64, 128, 256):      # the call picks the block rows itself; any choice must fit
+        g = max(lib.awqmi_moe_gemm_workspace_bytes(n, E, H, 2 * I, 0, tile),
+                lib.awqmi_moe_gemm_workspace_bytes(n, E, I, H, 0, tile))
+        cap = lib.awqmi_moe_align_capacity(n, E, tile)
+        payloads.append(g + 2 * n * 4 + cap * 4 + cap // tile * 4 + 4 + n * 2 * I * 2 + n * I * 2 + n * H * 2)
+    assert max(payloads) <= total <= max(payloads) + 9 * 256
     assert lib.awqmi_fused_moe_workspace_bytes(0, H, I, E, topk) == 0
     assert lib.awqmi_fused_moe_workspace_bytes(T, H, 100, E, topk) == 0
 
