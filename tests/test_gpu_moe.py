@@ -136,7 +136,9 @@ def test_moe_grouped_gemm_mfma_blocks(sba, gpu, bs, T, E, topk, K, N, G):
     assert awq_ref.rel_frobenius(y2, ref2) <= TOL
 
 
-@pytest.mark.parametrize("T,H,E,topk,I", [(2048, 2048, 128, 8, 768), (1024, 1024, 8, 2, 2048)])
+@pytest.mark.parametrize("T,H,E,topk,I", [(2048, 2048, 128, 8, 768), (1024, 1024, 8, 2, 2048),
+                                          (4096, 512, 4, 2, 384),     # many rows per expert
+                                          (640, 256, 4, 1, 1152)])    # top-1
 def test_fused_call_on_prefill_batches(sba, gpu, T, H, E, topk, I):
     """Batches with many slots per expert, where the one-call path takes the MFMA blocks:
     against the dense expert path and against the step-by-step path over 16-row blocks."""
