@@ -3,15 +3,39 @@
 // GEMMs, and the final sum over a token's slots.  All are latency-sized integer / elementwise
 // work; the expert GEMMs themselves are the MOE instantiation of the skinny kernel.
 #pragma once
+#include <type_traits>
 #include "awq_common.hpp"
 
 namespace awqmi {
+
+// Wave-wide max / sum by DPP row shifts and row broadcasts (full-rate VALU, no LDS crossbar
+// trips); the result is taken from lane 63 and returned wave-uniform.
+template <bool IS_MAX>
+__device__ __forceinline__ float wave_reduce_f32(float v) {
+  const int ident = IS_MAX ? (int)0xff800000u : 0;   // -inf / 0.0f
+  auto step = [&](auto CTRL, auto ROWS) {
+    const int o = __builtin_amdgcn_update_dpp(ident, __builtin_bit_cast(int, v), decltype(CTRL)::value,
+                                              decltype(ROWS)::value, 0xf, false);
+    const float f = __builtin_bit_cast(float, o);
+    v = IS_MAX ? fmaxf(v, f) : v + f;
+  };
+  using std::integral_constant;
+  step(integral_constant<int, 0x111>{}, integral_constant<int, 0xf>{});   // row_shr:1
+  step(integral_constant<int, 0x112>{}, integral_constant<int, 0xf>{});   // row_shr:2
+  step(integral_constant<int, 0x114>{}, integral_constant<int, 0xf>{});   // row_shr:4
+  step(integral_constant<int, 0x118>{}, integral_constant<int, 0xf>{});   // row_shr:8: lane 15 of a row = row total
+  step(integral_constant<int, 0x142>{}, integral_constant<int, 0xa>{});   // row_bcast:15 into rows 1, 3
+  step(integral_constant<int, 0x143>{}, integral_constant<int, 0xc>{});   // row_bcast:31 into rows 2, 3
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
 
 // One wave per token.  PER = experts per lane (E <= 64 * PER).
 // SIGMOID = false: softmax scores; selection runs on the raw logits (softmax is monotonic).
 // SIGMOID = true: score = sigmoid(logit); selection runs on score + bias[e] (bias may be
 // null), the weight is the score itself.  Ties go to the lowest expert id.  Weights are
 // optionally renormalised over the selected experts and multiplied by `scale`.
+// Each pick is one wave-wide max of the remaining keys, then a ballot of the lanes that hold
+// it (lowest expert id first); the winner's id and key are wave-uniform from there on.
 template <int PER, bool SIGMOID>
 __global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__ logits,
                                                        const float* __restrict__ bias, int T, int E,
@@ -22,10 +46,12 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__
   if (t >= T) return;
   float v[PER];      // selection key
   float sc[PER];     // score (SIGMOID only)
-  float mx = -INFINITY;
+  bool open[PER];    // expert exists and is not picked yet
+  float lmax = -INFINITY;
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int e = lane + 64 * i;
+    open[i] = e < E;
     const float x = e < E ? logits[(size_t)t * E + e] : -INFINITY;
     if (SIGMOID) {
       sc[i] = 1.f / (1.f + __expf(-x));
@@ -33,47 +59,47 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__
     } else {
       sc[i] = 0.f;
       v[i] = x;
-      mx = fmaxf(mx, x);
+      lmax = fmaxf(lmax, x);
     }
   }
-  float sum = 1.f;
+  float mx = 0.f, sum = 1.f;
   if (!SIGMOID) {
+    mx = wave_reduce_f32<true>(lmax);
+    float ls = 0.f;
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-    sum = 0.f;
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int e = lane + 64 * i;
-      if (e < E) sum += __expf(v[i] - mx);
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    for (int i = 0; i < PER; ++i)
+      if (lane + 64 * i < E) ls += __expf(v[i] - mx);
+    sum = wave_reduce_f32<false>(ls);
   }
 
   float sel_sum = 0.f;
   float my_w = 0.f;   // lane j keeps the weight of pick j (topk <= 64)
   int my_id = 0;
   for (int it = 0; it < topk; ++it) {
-    float best = -INFINITY, bsc = 0.f;
-    int bidx = 0x7fffffff;
+    float loc = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int e = lane + 64 * i;
-      if (e < E && (v[i] > best)) { best = v[i]; bidx = e; bsc = sc[i]; }   // ascending e: first max wins
+    for (int i = 0; i < PER; ++i)
+      if (open[i]) loc = fmaxf(loc, v[i]);
+    const float best = wave_reduce_f32<true>(loc);
+    int bidx = E;                                    // stays E only if every key left is NaN
+#pragma unroll
+    for (int i = PER - 1; i >= 0; --i) {             // descending, so the lowest id wins
+      const unsigned long long b = __ballot(open[i] && v[i] == best);
+      if (b) bidx = 64 * i + __builtin_ctzll(b);
     }
+    float bsc = 0.f;
+    if (SIGMOID) {
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ob = __shfl_xor(best, o);
-      const int oi = __shfl_xor(bidx, o);
-      const float os = SIGMOID ? __shfl_xor(bsc, o) : 0.f;
-      if (ob > best || (ob == best && oi < bidx)) { best = ob; bidx = oi; bsc = os; }
+      for (int i = 0; i < PER; ++i)
+        if ((bidx >> 6) == i)
+          bsc = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sc[i]), bidx & 63));
     }
     const float pw = SIGMOID ? bsc : __expf(best - mx) / sum;
     sel_sum += pw;
     if (lane == it) { my_w = pw; my_id = bidx; }
 #pragma unroll
     for (int i = 0; i < PER; ++i)
-      if (lane + 64 * i == bidx) v[i] = -INFINITY;
+      if (lane + 64 * i == bidx) open[i] = false;
   }
   if (lane < topk) {
     ids[(size_t)t * topk + lane] = my_id;
@@ -239,10 +265,22 @@ __global__ __launch_bounds__(256) void moe_sum_kernel(const half_t* __restrict__
   if (idx >= (size_t)T * per_row) return;
   const size_t t = idx / per_row, c = (idx % per_row) * 8;
   float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int j = 0; j < topk; ++j) {
-    const h8 v = *reinterpret_cast<const h8*>(in + (t * topk + j) * H + c);
+  // eight slot rows in flight at a time (a loop of single loads pays one memory round trip
+  // per slot); the sum runs in slot order either way
+  for (int j0 = 0; j0 < topk; j0 += 8) {
+    h8 v[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) s[i] += (float)v[i];
+    for (int u = 0; u < 8; ++u) {
+      const int j = min(j0 + u, topk - 1);
+      v[u] = *reinterpret_cast<const h8*>(in + (t * topk + j) * H + c);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (j0 + u < topk) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s[i] += (float)v[u][i];
+      }
+    }
   }
   h8 o;
 #pragma unroll
