@@ -131,6 +131,37 @@ MfmaPlan plan_mfma(int M, int K, int N) {
 
 }  // namespace
 
+// softmax routing and align in one launch (at most 16 tokens); same results as the two calls
+template <int P>
+static int moe_route_align_launch(const float* logits, int T, int E, int topk, int renormalize,
+                                  int32_t* ids, float* wts, int tile_m, int cap, int32_t* sorted,
+                                  int32_t* experts, int32_t* npp, hipStream_t st) {
+  static std::atomic<bool> attr{false};     // one flag per instantiation
+  if (!attr.load(std::memory_order_acquire)) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(moe_route_align_kernel<P, false>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             (MOE_ALIGN_WAVES + 2) * AWQMI_MAX_EXPERTS * (int)sizeof(int));
+    if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
+    attr.store(true, std::memory_order_release);
+  }
+  hipLaunchKernelGGL((moe_route_align_kernel<P, false>), dim3(1), dim3(1024),
+                     (size_t)(MOE_ALIGN_WAVES + 2) * E * sizeof(int), st, logits, (const float*)nullptr, T, E,
+                     topk, renormalize, 1.f, ids, wts, tile_m, cap, sorted, experts, npp);
+  return launch_status();
+}
+
+static int moe_route_align_small(const float* logits, int T, int E, int topk, int renormalize,
+                                 int32_t* ids, float* wts, int tile_m, int32_t* sorted, int32_t* experts,
+                                 int32_t* npp, void* stream) {
+  const int cap = (int)awqmi_moe_align_capacity(T * topk, E, tile_m);
+  hipStream_t st = (hipStream_t)stream;
+  if (E <= 64) return moe_route_align_launch<1>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
+  if (E <= 128) return moe_route_align_launch<2>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
+  if (E <= 256) return moe_route_align_launch<4>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
+  if (E <= 512) return moe_route_align_launch<8>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
+  return moe_route_align_launch<16>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
+}
+
 extern "C" {
 
 int awqmi_version(void) { return AWQMI_VERSION; }
@@ -443,12 +474,22 @@ size_t awqmi_moe_gemm_workspace_bytes(int n_slots, int E, int K, int N, int spli
 // Can the w13 GEMM of a block write silu(gate) * up itself?  Needs the paired-column launch
 // (two column blocks per workgroup: the gate block and its up block), i.e. no split across
 // workgroups, an even chunk count, [gate | up] halves that are whole column blocks, and
-// enough blocks that the halved workgroup count still fills the chip.
+// enough blocks that the halved workgroup count still fills the chip.  It pays from about
+// eight real rows per 16-row block on (measured on 2048 x 1536 experts, 128 of them: 6 %
+// faster at 12 rows per block, 3 - 5 % slower at 2 - 6); below that the separate activation
+// kernel is cheaper than the two-waves-per-column-block form of the GEMM.
 static bool moe_can_fuse_act(int n_slots, int E, int K, int N) {
   const MoePlan pl = moe_plan(n_slots, E, K, N, 16, 0);
   const long long live_blocks = std::max<long long>((n_slots + 15) / 16, std::min(n_slots, E));
   return pl.wpl == 2 && pl.split == 1 && K % 128 == 0 && (K / 128) % 2 == 0 && N % 512 == 0 &&
-         live_blocks * (pl.ncb / 2) >= 256;
+         live_blocks * (pl.ncb / 2) >= 256 && n_slots >= 8 * live_blocks;
+}
+
+// Same question for a launch that is split in K: the last arrivers of a gate block and its up
+// block finish both and apply the activation.
+static bool moe_can_fuse_act_split(int n_slots, int E, int K, int N) {
+  const MoePlan pl = moe_plan(n_slots, E, K, N, 16, 0);
+  return pl.wpl == 2 && pl.split > 1 && N % 512 == 0 && pl.ncb % 2 == 0;
 }
 
 static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
@@ -574,14 +615,21 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   const long long live_blocks = std::max<long long>((n_slots + 15) / 16, std::min(n_slots, E));
   const bool pair_cols = tile_m == 16 && wpl == 2 && split == 1 && K / 128 <= 8 && (K / 128) % 2 == 0 &&
                          live_blocks * ((ncb + 1) / 2) >= 256 && !(variant >= 0 && (variant & 64));
-  if (fuse_act && (split != 1 || wpl != 2 || tile_m != 16 || ncb % 2 != 0 || (K / 128) % 2 != 0))
+  // fused activation: without a split the paired-column kernel (gate and up block in one
+  // workgroup); with a split the ordinary launch whose last arrivers pair the blocks up
+  if (fuse_act && (wpl != 2 || tile_m != 16 || ncb % 2 != 0 || N % 512 != 0 ||
+                   (split == 1 && (K / 128) % 2 != 0)))
     return AWQMI_BAD_ARGUMENT;
-  const int ncg = fuse_act ? ncb / 2 : (pair_cols ? (ncb + 1) / 2 : ncb);
+  const bool act_split = fuse_act && split > 1;
+  p.act_split = act_split ? 1 : 0;
+  const bool act_pair = fuse_act && split == 1;
+  const int ncg = act_pair ? ncb / 2 : (pair_cols ? (ncb + 1) / 2 : ncb);
   // runs of grp slots, dealt to the 8 XCDs in turn; the last deal may be partial
   const long long runs = (long long)(nblk / p.grp) * ncg * split;
   const dim3 grid((unsigned)((runs + 7) / 8 * 8 * p.grp));
   hipStream_t st = (hipStream_t)stream;
-  if (fuse_act) launch_gemv<2, 1, true, 2, 2, true>(p, grid, st);
+  if (act_pair) launch_gemv<2, 1, true, 2, 2, true>(p, grid, st);
+  else if (act_split) launch_gemv<2, 1, true, 2>(p, grid, st);
   else if (tile_m == 32) launch_gemv<2, 2, true>(p, grid, st);
   else if (wpl == 2 && variant >= 0 && (variant & 2)) launch_gemv<2, 1, true, 4>(p, grid, st);
   else if (pair_cols) launch_gemv<2, 1, true, 2, 2>(p, grid, st);
@@ -712,15 +760,28 @@ int awqmi_fused_moe_f16(const void* hidden, const float* router_logits, const in
   void* h13 = ws + L.h13;
   void* act = ws + L.act;
   void* o = ws + L.o;
-  int st = awqmi_moe_topk_softmax_f32(router_logits, T, E, topk, renormalize, ids, wts, stream);
-  if (st) return st;
-  st = awqmi_moe_align(ids, L.n_slots, E, tile, sorted, experts, npp, stream);
-  if (st) return st;
+  int st;
+  if (T <= MOE_ALIGN_WAVES) {
+    st = moe_route_align_small(router_logits, T, E, topk, renormalize, ids, wts, tile, sorted, experts, npp, stream);
+    if (st) return st;
+  } else {
+    st = awqmi_moe_topk_softmax_f32(router_logits, T, E, topk, renormalize, ids, wts, stream);
+    if (st) return st;
+    st = awqmi_moe_align(ids, L.n_slots, E, tile, sorted, experts, npp, stream);
+    if (st) return st;
+  }
   const int Gn = norm_group(H, group);
   if (tile == 16 && gemv_tiled_ok(H, Gn) && moe_can_fuse_act(L.n_slots, E, H, 2 * inter) &&
       !(g_gemv_variant.load(std::memory_order_relaxed) >= 0 &&
         (g_gemv_variant.load(std::memory_order_relaxed) & 1024))) {
     // the w13 GEMM writes silu(gate) * up itself
+    st = moe_gemm_impl(hidden, w13_q, w13_s, w13_z, act, sorted, experts, npp, nullptr, L.n_slots, topk, 16, E, H,
+                       2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream, true);
+    if (st) return st;
+  } else if (tile == 16 && gemv_tiled_ok(H, Gn) && moe_can_fuse_act_split(L.n_slots, E, H, 2 * inter) &&
+             !(g_gemv_variant.load(std::memory_order_relaxed) >= 0 &&
+               (g_gemv_variant.load(std::memory_order_relaxed) & 1024))) {
+    // few blocks: the w13 GEMM is split in K and its last arrivers write silu(gate) * up
     st = moe_gemm_impl(hidden, w13_q, w13_s, w13_z, act, sorted, experts, npp, nullptr, L.n_slots, topk, 16, E, H,
                        2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream, true);
     if (st) return st;

@@ -42,6 +42,8 @@ struct GemvParams {
   int ldy;      // elements between output rows (N, or N / 2 when the activation is fused)
   int nblk;     // sorted-token blocks covered by the launch (a multiple of grp)
   int grp;      // sorted-token blocks per XCD run
+  int act_split; // split-K launch over [gate | up] columns: the last arriver of a gate block and
+                 // its up block writes silu(gate) * up (one 16-row block, four waves per column block)
   long long w_stride, s_stride, z_stride;  // elements per expert
 };
 
@@ -429,12 +431,12 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
     }
   };
   // gate tile in red[0], up tile in red[1] -> silu(gate) * up, 16 bytes per thread
-  auto emit_act = [&](int rows) {
+  auto emit_act = [&](int rows, int cbo) {
     constexpr int WPB = 16 * WPL;
     for (int it = tid; it < rows * WPB; it += 256) {
       const int m = it / WPB, wl = it % WPB;
       const int jj = wl / WPL, ww = wl % WPL;
-      const int col = cb * CB + wl * 8;
+      const int col = cbo * CB + wl * 8;
       const int sid = s_sid[m];
       if (sid >= p.n_slots) continue;
       h8 o;
@@ -474,7 +476,7 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
       }
       __syncthreads();
       if (ACT) {
-        emit_act(rows);
+        emit_act(rows, cb);
       } else {
         emit(mb, rows, false, 0, cb * 2);
         if (cb * 2 + 1 < p.ncb) emit(mb, rows, false, 1, cb * 2 + 1);
@@ -526,14 +528,21 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
   // before its arrival is counted; whoever arrives last sums all partials in fixed order.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  if (tid == 0) s_last = (atomicAdd(p.cnt + tile, 1) == p.split_k - 1);
+  // fused activation: a gate block and its up block (half the column blocks further on) share
+  // one counter, and the last of their 2 x split workgroups finishes both tiles
+  const bool acts = MOE && MB == 1 && KW == 4 && !ACT && p.act_split;
+  const int hcb = p.ncb / 2;
+  const int cbg = acts ? cb % hcb : cb;
+  const size_t ctile = acts ? (size_t)blk * hcb + cbg : tile;
+  const int arrivals = acts ? 2 * p.split_k : p.split_k;
+  if (tid == 0) s_last = (atomicAdd(p.cnt + ctile, 1) == arrivals - 1);
   __syncthreads();
   if (!s_last) return;
   const size_t sstride = ntiles * MB * TILE_F;
   // U pairs per thread x 8 parts per batch: 8 * U independent 8-byte loads in flight; parts
   // are added in index order whatever the arrival order was.  Out-of-range slots read a valid
   // address and are dropped by a select, so no load sits behind a branch.
-  auto finish = [&](auto u_tag, const float* base, int nelem) {
+  auto finish = [&](auto u_tag, const float* base, int nelem, int buf = 0) {
     constexpr int U = decltype(u_tag)::value;
     constexpr int SU = 8;
     f2 v[U];
@@ -561,8 +570,26 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (idx[u] < nelem) *reinterpret_cast<f2*>(&red[0][idx[u] / (NT * 16)][idx[u] % (NT * 16)]) = v[u];
+      if (idx[u] < nelem) *reinterpret_cast<f2*>(&red[buf][idx[u] / (NT * 16)][idx[u] % (NT * 16)]) = v[u];
   };
+  if (acts) {
+    const int rows = min(16, rows_total);
+    const int nelem = rows * (NT * 16);
+    if (nelem > 0) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const float* base = p.part + ((size_t)blk * p.ncb + cbg + half * hcb) * TILE_F;
+        if (nelem <= 512) finish(std::integral_constant<int, 1>{}, base, nelem, half);
+        else if (nelem <= 1024) finish(std::integral_constant<int, 2>{}, base, nelem, half);
+        else if (nelem <= 2048) finish(std::integral_constant<int, 4>{}, base, nelem, half);
+        else finish(std::integral_constant<int, 8>{}, base, nelem, half);
+      }
+    }
+    __syncthreads();
+    emit_act(rows, cbg);
+    if (tid == 0) __hip_atomic_store(p.cnt + ctile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return;
+  }
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int rows = min(16, max(0, rows_total - 16 * mb));

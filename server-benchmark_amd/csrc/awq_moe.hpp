@@ -37,13 +37,11 @@ __device__ __forceinline__ float wave_reduce_f32(float v) {
 // Each pick is one wave-wide max of the remaining keys, then a ballot of the lanes that hold
 // it (lowest expert id first); the winner's id and key are wave-uniform from there on.
 template <int PER, bool SIGMOID>
-__global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__ logits,
-                                                       const float* __restrict__ bias, int T, int E,
-                                                       int topk, int renorm, float scale,
-                                                       int* __restrict__ ids, float* __restrict__ wts) {
+__device__ __forceinline__ void moe_topk_token(const float* __restrict__ logits,
+                                               const float* __restrict__ bias, int t, int E, int topk,
+                                               int renorm, float scale, int* __restrict__ ids,
+                                               float* __restrict__ wts) {
   const int lane = threadIdx.x & 63;
-  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (t >= T) return;
   float v[PER];      // selection key
   float sc[PER];     // score (SIGMOID only)
   bool open[PER];    // expert exists and is not picked yet
@@ -107,6 +105,16 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__
   }
 }
 
+template <int PER, bool SIGMOID>
+__global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__ logits,
+                                                       const float* __restrict__ bias, int T, int E,
+                                                       int topk, int renorm, float scale,
+                                                       int* __restrict__ ids, float* __restrict__ wts) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  moe_topk_token<PER, SIGMOID>(logits, bias, t, E, topk, renorm, scale, ids, wts);
+}
+
 // Single workgroup of 16 waves.  Dynamic LDS: cnt[16][E] + padded[E] + start[E].
 // Wave w owns the contiguous slice [w*seg, (w+1)*seg) of the flat slot list, so placing
 // slices in wave order and slots in index order inside a slice gives a stable sort.  Inside a
@@ -115,12 +123,10 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__
 // position per (wave, expert) lives in LDS and is bumped by one LDS atomic per slot after all
 // lanes of the batch have read it.
 constexpr int MOE_ALIGN_WAVES = 16;
-__global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int n, int E,
-                                                         int tile_m, int cap,
-                                                         int* __restrict__ sorted,
-                                                         int* __restrict__ expert_ids,
-                                                         int* __restrict__ npp) {
-  extern __shared__ int sm[];
+__device__ __forceinline__ void moe_align_block(const int* __restrict__ ids, int n, int E, int tile_m,
+                                                int cap, int* __restrict__ sorted,
+                                                int* __restrict__ expert_ids, int* __restrict__ npp,
+                                                int* sm) {
   constexpr int NWV = MOE_ALIGN_WAVES;
   int* cnt = sm;               // [NWV][E], later the running write position
   int* padded = sm + NWV * E;  // [E]
@@ -236,6 +242,33 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
       if (c0 + 64 * b < se) place(c0 + 64 * b + lane, more[b]);
     }
   }
+}
+
+__global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int n, int E,
+                                                         int tile_m, int cap,
+                                                         int* __restrict__ sorted,
+                                                         int* __restrict__ expert_ids,
+                                                         int* __restrict__ npp) {
+  extern __shared__ int sm[];
+  moe_align_block(ids, n, E, tile_m, cap, sorted, expert_ids, npp, sm);
+}
+
+// Routing and align in one launch for batches of at most 16 tokens (one wave per token, the
+// same single workgroup then sorts the T * topk slots): a decode step of a few sequences
+// spends more on the second launch than on either kernel's work.
+template <int PER, bool SIGMOID>
+__global__ __launch_bounds__(1024) void moe_route_align_kernel(const float* __restrict__ logits,
+                                                               const float* __restrict__ bias, int T,
+                                                               int E, int topk, int renorm, float scale,
+                                                               int* ids, float* __restrict__ wts, int tile_m,
+                                                               int cap, int* __restrict__ sorted,
+                                                               int* __restrict__ expert_ids,
+                                                               int* __restrict__ npp) {
+  extern __shared__ int sm[];
+  const int wave = threadIdx.x >> 6;
+  if (wave < T) moe_topk_token<PER, SIGMOID>(logits, bias, wave, E, topk, renorm, scale, ids, wts);
+  __syncthreads();   // the ids written above are read back by the same workgroup
+  moe_align_block(ids, T * topk, E, tile_m, cap, sorted, expert_ids, npp, sm);
 }
 
 __global__ __launch_bounds__(256) void silu_and_mul_kernel(const half_t* __restrict__ in,

@@ -259,9 +259,11 @@ def test_moe_odd_shapes_vs_dense_expert_path(sba, gpu, T, H, E, topk, I):
     assert float((y16.float() - ref).norm() / ref.norm()) <= TOL
 
 
-@pytest.mark.parametrize("T", [128, 512])
+@pytest.mark.parametrize("T", [1, 4, 128, 512])
 def test_fused_activation_agrees_with_step_by_step(sba, gpu, T):
-    """Block sizes at which the w13 GEMM of the one-call path writes silu(gate) * up itself.  Its
+    """Block sizes at which the w13 GEMM of the one-call path writes silu(gate) * up itself (T = 1, 4:
+    split in K, the last arrivers of a gate block and its up block apply it; 128, 512: gate and up
+    block in one workgroup).  Its
     two waves per column block add K in another order than the four of the separate-kernel
     path, so the two agree to fp32 summation order (a few last-bit differences after the fp16
     roundings), not bit for bit; both must meet the tolerance against the dense expert path."""
