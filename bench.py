@@ -459,6 +459,20 @@ def main():
                           "cpu_ms_median": round(cpu_ts[len(cpu_ts) // 2] * 1e3, 2), "cpu_threads": nthreads,
                           "gpu_vs_cpu_rel_frobenius": round(err0, 6)}
         worst = max(worst, err0)
+        # one prefill point on the CPU path (o_proj, M = 512: 69 GFLOP; larger ones take minutes)
+        n0, K0, N0 = layers[1]
+        xp = torch.randn((512, K0), generator=torch.Generator().manual_seed(512), dtype=torch.float32).half()
+        qw, sc, qz = (t.cpu() for t in W[n0][0])
+        t1 = time.perf_counter()
+        ycp = awq_ref.cpu_linear_torch(xp, qw, sc, qz, G)
+        cpu_p = time.perf_counter() - t1
+        ygp = sba.awq_gemm(xp.to(dev), *W[n0][0], 0).float().cpu()
+        errp = float((ygp - ycp.float()).norm() / ycp.float().norm())
+        worst = max(worst, errp)
+        cpu_prefill = {"layer": n0, "M": 512, "cpu_ms": round(cpu_p * 1e3, 1),
+                       "cpu_TFLOPs": round(2.0 * 512 * K0 * N0 / cpu_p / 1e12, 4),
+                       "gpu_vs_cpu_rel_frobenius": round(errp, 6)}
+        del qw, sc, qz, ycp, ygp
         cpu_model = ""
         try:
             with open("/proc/cpuinfo") as f:
@@ -472,7 +486,8 @@ def main():
                                "cores": nthreads, "kind": "port",
                                "sample": f"two passes over the 16 calls of one step, one PyTorch dequantize+matmul "
                                          f"call each: {len(sample)} calls, {sample_t:.1f} s total",
-                               "cpu": cpu_model, "gpu_vs_cpu_rel_frobenius_max": round(worst, 6)}
+                               "cpu": cpu_model, "prefill_point": cpu_prefill,
+                               "gpu_vs_cpu_rel_frobenius_max": round(worst, 6)}
         log(f"[bench] cpu baseline {out['cpu_baseline']['value']} GB/s on {nthreads} threads; "
             f"GPU vs CPU rel. Frobenius max {worst:.2e}")
         if worst > 2e-3:
