@@ -151,6 +151,10 @@ int awqmi_moe_sum_f16(const void* in_f16, void* out_f16, int T, int topk, int H,
  * zero-initialised once; the call itself allocates nothing and is safe to capture in a HIP
  * graph.  H and inter must be multiples of 128 with group in {32, 64, 128 * i}. */
 size_t awqmi_fused_moe_workspace_bytes(int T, int H, int inter, int E, int topk);
+/* Sorted-token block rows awqmi_fused_moe_f16 uses for these shapes: 16 (skinny kernel) or
+ * 64 / 128 / 256 (MFMA kernel, prefill-sized batches).  A query like awqmi_gemm_auto_split_k;
+ * 0 for shapes the call would refuse. */
+int awqmi_fused_moe_block_rows(int T, int H, int inter, int E, int topk, int group);
 int awqmi_fused_moe_f16(const void* hidden_f16, const float* router_logits, const int32_t* w13_qweight,
                         const void* w13_scales_f16, const int32_t* w13_qzeros,
                         const int32_t* w2_qweight, const void* w2_scales_f16, const int32_t* w2_qzeros,

@@ -32,6 +32,7 @@ SIGNATURES = {
     "awqmi_silu_and_mul_f16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "awqmi_moe_sum_f16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "awqmi_fused_moe_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "awqmi_fused_moe_block_rows": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "awqmi_fused_moe_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t,
                                     c_void_p]),

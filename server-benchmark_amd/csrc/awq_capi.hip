@@ -736,6 +736,12 @@ size_t awqmi_fused_moe_workspace_bytes(int T, int H, int inter, int E, int topk)
   return most;
 }
 
+int awqmi_fused_moe_block_rows(int T, int H, int inter, int E, int topk, int group) {
+  if (T <= 0 || H <= 0 || inter <= 0 || E <= 0 || H % 8 != 0 || inter % 8 != 0) return 0;
+  if (topk <= 0 || topk > E || topk > 64 || E > AWQMI_MAX_EXPERTS || (long long)T * topk > (1LL << 30)) return 0;
+  return moe_pick_tile(T * topk, E, H, inter, group);
+}
+
 int awqmi_fused_moe_f16(const void* hidden, const float* router_logits, const int32_t* w13_q,
                         const void* w13_s, const int32_t* w13_z, const int32_t* w2_q, const void* w2_s,
                         const int32_t* w2_z, void* out, int T, int H, int inter, int E, int topk,

@@ -88,6 +88,26 @@ def test_fused_moe_workspace_covers_every_intermediate(lib):
     assert lib.awqmi_fused_moe_workspace_bytes(T, H, 100, E, topk) == 0
 
 
+def test_fused_moe_block_rows(lib):
+    """Block rows the one-call MoE entry picks: the skinny kernel's 16 for decode-sized batches,
+    the MFMA kernel's 64 / 128 / 256 where measurements favoured them (points of the fit)."""
+    q = lib.awqmi_fused_moe_block_rows
+    for T in (1, 16, 128, 512, 1024):
+        assert q(T, 2048, 768, 128, 8, 128) == 16
+    assert q(2048, 2048, 768, 128, 8, 128) == 128
+    assert q(4096, 2048, 768, 128, 8, 128) == 128
+    assert q(512, 6144, 2560, 160, 8, 128) == 16
+    assert q(1024, 6144, 2560, 160, 8, 128) == 64
+    assert q(2048, 6144, 2560, 160, 8, 128) == 128
+    assert q(8192, 6144, 2560, 160, 8, 128) == 256
+    assert q(64, 4096, 14336, 8, 2, 128) == 16
+    assert q(1024, 4096, 14336, 8, 2, 128) in (128, 256)
+    assert q(4096, 2048, 776, 128, 8, 128) == 16       # inter no multiple of 128: MFMA form not available
+    assert q(0, 2048, 768, 128, 8, 128) == 0 and q(4, 2048, 768, 128, 200, 128) == 0
+    for T in (1, 100, 5000):                           # every choice fits the workspace the query sizes
+        assert lib.awqmi_fused_moe_workspace_bytes(T, 2048, 768, 128, 8) > 0
+
+
 def test_workspace_and_split_k_queries(lib):
     for M, K, N in [(1, 8192, 10240), (16, 8192, 8192), (16, 8192, 59136), (4, 29568, 8192), (8, 4096, 4096)]:
         s = lib.awqmi_gemm_auto_split_k(M, K, N, 128)
