@@ -15,7 +15,8 @@
  *     8c + {0,2,4,6,1,3,5,7}[i].  W[k,n] = fp16((w - z) * s), one rounding.
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
  *   - Every call validates on the host first and launches nothing on error; calls are
- *     asynchronous, never synchronise, never allocate and never keep a pointer.
+ *     asynchronous, never synchronise, never allocate and never keep a pointer, and can be
+ *     captured in a HIP graph (grid sizes depend on shapes only).
  *   - Return value: AWQMI_OK or one of the awqmi_status codes below.
  */
 #ifndef AWQ_MI355X_H
@@ -44,6 +45,12 @@ typedef enum awqmi_status {
 #define AWQMI_MAX_SPLIT_K 64
 #define AWQMI_MAX_EXPERTS 1024
 
+/* Optional one-time set-up on the current device: raises the dynamic-LDS limit of the kernels
+ * that need it.  Every entry point does the same on its first use; call this once after
+ * loading the library if the first use may sit inside a stream capture.  The library assumes
+ * one GPU per process (the harness starts one server process per replica and GPU set,
+ * reference utils/generate_compose.py:85-100). */
+int awqmi_init(void);
 int awqmi_version(void);
 const char* awqmi_status_string(int status);
 /* hipError_t of the last AWQMI_LAUNCH_FAILED on the calling thread (0 if none). */

@@ -12,6 +12,7 @@ c_int, c_void_p, c_size_t = ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 
 # name -> (restype, argtypes); mirrors include/awq_mi355x.h one to one
 SIGNATURES = {
+    "awqmi_init": (c_int, []),
     "awqmi_version": (c_int, []),
     "awqmi_status_string": (ctypes.c_char_p, [c_int]),
     "awqmi_last_hip_error": (c_int, []),

@@ -131,19 +131,45 @@ MfmaPlan plan_mfma(int M, int K, int N) {
 
 }  // namespace
 
+// Kernels that use more dynamic LDS than the default limit need a function attribute; it is
+// set once per process for all of them (by awqmi_init, or by the first call that needs one).
+static int ensure_kernel_attributes() {
+  static std::atomic<bool> done{false};
+  if (done.load(std::memory_order_acquire)) return AWQMI_OK;
+  const void* mfma[] = {
+      reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1, 8>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1, 8>),
+      reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 2, 8>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 2, 8>),
+      reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1>),
+      reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 2>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 2>),
+      reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 3>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 3>),
+      reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 4>),
+      reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1, 8, true>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1, 8, true>),
+      reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 2, 8, true>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 2, 8, true>),
+      reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4, 4, true>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 4, 4, true>)};
+  for (const void* fn : mfma) {
+    const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, PF_LDS_BYTES);
+    if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
+  }
+  const void* align[] = {
+      reinterpret_cast<const void*>(moe_align_kernel),
+      reinterpret_cast<const void*>(moe_route_align_kernel<1, false>), reinterpret_cast<const void*>(moe_route_align_kernel<2, false>),
+      reinterpret_cast<const void*>(moe_route_align_kernel<4, false>), reinterpret_cast<const void*>(moe_route_align_kernel<8, false>),
+      reinterpret_cast<const void*>(moe_route_align_kernel<16, false>)};
+  for (const void* fn : align) {
+    const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             (MOE_ALIGN_WAVES + 2) * AWQMI_MAX_EXPERTS * (int)sizeof(int));
+    if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
+  }
+  done.store(true, std::memory_order_release);
+  return AWQMI_OK;
+}
+
 // softmax routing and align in one launch (at most 16 tokens); same results as the two calls
 template <int P>
 static int moe_route_align_launch(const float* logits, int T, int E, int topk, int renormalize,
                                   int32_t* ids, float* wts, int tile_m, int cap, int32_t* sorted,
                                   int32_t* experts, int32_t* npp, hipStream_t st) {
-  static std::atomic<bool> attr{false};     // one flag per instantiation
-  if (!attr.load(std::memory_order_acquire)) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(moe_route_align_kernel<P, false>),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             (MOE_ALIGN_WAVES + 2) * AWQMI_MAX_EXPERTS * (int)sizeof(int));
-    if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
-    attr.store(true, std::memory_order_release);
-  }
+  if (int st = ensure_kernel_attributes()) return st;
   hipLaunchKernelGGL((moe_route_align_kernel<P, false>), dim3(1), dim3(1024),
                      (size_t)(MOE_ALIGN_WAVES + 2) * E * sizeof(int), st, logits, (const float*)nullptr, T, E,
                      topk, renormalize, 1.f, ids, wts, tile_m, cap, sorted, experts, npp);
@@ -163,6 +189,8 @@ static int moe_route_align_small(const float* logits, int T, int E, int topk, in
 }
 
 extern "C" {
+
+int awqmi_init(void) { return ensure_kernel_attributes(); }
 
 int awqmi_version(void) { return AWQMI_VERSION; }
 
@@ -299,26 +327,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   // 32-bit, so every operand must stay below 4 GiB
   const bool pow2g = (G & (G - 1)) == 0 && G >= 8;
   if (mfma_ok) {
-    static std::atomic<bool> attr_set{false};
-    if (!attr_set.load(std::memory_order_acquire)) {
-      const void* fns[12] = {reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1, 8>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1, 8>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 2, 8>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 2, 8>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 4>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 3>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 3>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 2>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 2>)};
-      for (const void* fn : fns) {
-        const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, PF_LDS_BYTES);
-        if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
-      }
-      attr_set.store(true, std::memory_order_release);
-    }
+    if (int st = ensure_kernel_attributes()) return st;
     const int slab = mfma_slab_rows(M, K);
     for (int r0 = 0; r0 < M; r0 += slab) {
     const int Ms = M - r0 < slab ? M - r0 : slab;
@@ -415,14 +424,7 @@ int awqmi_moe_align(const int32_t* topk_ids, int n_slots, int E, int tile_m, int
   if (n_slots <= 0 || E <= 0) return AWQMI_BAD_SHAPE;
   if (E > AWQMI_MAX_EXPERTS || tile_m <= 0 || tile_m > 4096) return AWQMI_BAD_ARGUMENT;
   const int cap = (int)awqmi_moe_align_capacity(n_slots, E, tile_m);
-  static std::atomic<bool> align_attr{false};
-  if (!align_attr.load(std::memory_order_acquire)) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(moe_align_kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             (MOE_ALIGN_WAVES + 2) * AWQMI_MAX_EXPERTS * (int)sizeof(int));
-    if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
-    align_attr.store(true, std::memory_order_release);
-  }
+  if (int st = ensure_kernel_attributes()) return st;
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)(MOE_ALIGN_WAVES + 2) * E * sizeof(int),
                      (hipStream_t)stream, topk_ids, n_slots, E, tile_m, cap, sorted_token_ids,
                      expert_ids, num_tokens_post_padded);
@@ -534,20 +536,7 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
     if (x_rows * K * 2 >= (1ull << 32) || (size_t)K * NW * 4 >= (1ull << 32) ||
         (size_t)(K / G) * N * 2 >= (1ull << 32))
       return AWQMI_BAD_SHAPE;
-    static std::atomic<bool> gattr{false};
-    if (!gattr.load(std::memory_order_acquire)) {
-      const void* fns[6] = {reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1, 8, true>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1, 8, true>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 2, 8, true>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 2, 8, true>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 4, 4, true>),
-                            reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 4, 4, true>)};
-      for (const void* fn : fns) {
-        const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, PF_LDS_BYTES);
-        if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
-      }
-      gattr.store(true, std::memory_order_release);
-    }
+    if (int st = ensure_kernel_attributes()) return st;
     MfmaGemmParams p{};
     p.x = reinterpret_cast<const half_t*>(x);
     p.qw = reinterpret_cast<const uint32_t*>(qweight);

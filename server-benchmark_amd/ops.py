@@ -59,6 +59,10 @@ def get_workspace(device, nbytes: int) -> torch.Tensor:
            torch.cuda.current_stream(dev).cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if not _workspaces:
+            # first GPU use in this process: the library's one-time set-up, so that no later
+            # call (possibly inside a stream capture) has to do it
+            _lib.check(_lib.load().awqmi_init(), "awqmi_init")
         ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
         _workspaces[key] = ws
     return ws

@@ -88,6 +88,17 @@ def test_fused_moe_workspace_covers_every_intermediate(lib):
     assert lib.awqmi_fused_moe_workspace_bytes(T, H, 100, E, topk) == 0
 
 
+def test_init_without_a_gpu_reports_a_launch_failure(lib):
+    """awqmi_init needs a device; without one it returns a status (no abort, no exception)."""
+    import torch
+    st = lib.awqmi_init()
+    if torch.cuda.is_available():
+        assert st == 0
+    else:
+        assert st == 5 and lib.awqmi_last_hip_error() != 0
+        assert b"launch" in lib.awqmi_status_string(st).lower()
+
+
 def test_fused_moe_block_rows(lib):
     """Block rows the one-call MoE entry picks: the skinny kernel's 16 for decode-sized batches,
     the MFMA kernel's 64 / 128 / 256 where measurements favoured them (points of the fit)."""
