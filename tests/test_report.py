@@ -31,6 +31,40 @@ def test_reader_on_recorded_blocks(report, name):
     assert metrics == want
 
 
+REFERENCE_RESULTS = pathlib.Path("/root/reference/results")
+
+
+@pytest.mark.skipif(not REFERENCE_RESULTS.is_dir(), reason="the harness's recorded results are not on this machine")
+def test_reader_on_every_recorded_result_file(report):
+    """Every benchmark log the harness recorded: what the reader returns must agree with the
+    block's own totals (tokens and requests over the duration, read here line by line, not
+    through the reader's patterns) and with the latency lines."""
+    files = sorted(REFERENCE_RESULTS.glob("*/*_vllm_benchmark.txt"))
+    assert len(files) >= 20
+    checked = 0
+    for f in files:
+        text = f.read_text(errors="replace")
+        if "Serving Benchmark Result" not in text:
+            continue          # a run that failed before the result block
+        field = {}
+        for line in text.splitlines():
+            if ":" in line:
+                k, _, v = line.rpartition(":")
+                try:
+                    field[k.strip()] = float(v)
+                except ValueError:
+                    pass
+        total, m = report.parse_serving_result(text)
+        dur = field["Benchmark duration (s)"]
+        assert total == field["Total Token throughput (tok/s)"], f.name
+        assert total == pytest.approx((field["Total input tokens"] + field["Total generated tokens"]) / dur, rel=2e-3), f.name
+        assert m["output_throughput"] == pytest.approx(field["Total generated tokens"] / dur, rel=2e-3), f.name
+        assert m["request_throughput"] == pytest.approx(field["Successful requests"] / dur, abs=0.006), f.name
+        assert m["mean_ttft_ms"] == field["Mean TTFT (ms)"] and m["mean_tpot_ms"] == field["Mean TPOT (ms)"], f.name
+        checked += 1
+    assert checked >= 20
+
+
 def test_reader_without_total(report):
     assert report.parse_serving_result("Request throughput (req/s):   4.2\n") == (None, {})
     total, metrics = report.parse_serving_result("Total Token throughput (tok/s):   10.5\n")
