@@ -57,6 +57,68 @@ def test_gpu_plumbing_is_rocm(deploy, stack):
         deploy.compose(3, 4, 1, "c", "/m", "m", "/hf", total_gpus=8)
 
 
+REFERENCE_RESULTS = pathlib.Path("/root/reference/results")
+
+
+def _recorded_compose(text):
+    """The YAML of the "Docker Compose Configuration" block of a benchmark log, or None."""
+    head = "Docker Compose Configuration"
+    if head not in text:
+        return None
+    body = text.split(head, 1)[1].split("\n", 1)[1]
+    lines = []
+    for line in body.splitlines():
+        if line.startswith("====") or line.startswith("----"):
+            break
+        lines.append(line)
+    return yaml.safe_load("\n".join(lines))
+
+
+@pytest.mark.skipif(not REFERENCE_RESULTS.is_dir(), reason="the harness's recorded results are not on this machine")
+def test_every_recorded_stack(deploy):
+    """Every compose block the harness recorded, regenerated from its own parameters (instance
+    count, parallel sizes, model, extra arguments read off the block): same services, same
+    commands, ports, health checks, nginx and benchmark services, and each instance gets the GPU
+    indexes the recorded block reserved for it -- as HIP_VISIBLE_DEVICES instead of a
+    device reservation."""
+    files = sorted(REFERENCE_RESULTS.glob("*/*_vllm_benchmark.txt"))
+    checked = 0
+    for f in files:
+        doc = _recorded_compose(f.read_text(errors="replace"))
+        if not doc:
+            continue
+        want = doc["services"]
+        n = sum(1 for k in want if k.startswith("vllm_"))
+        cmd = want["vllm_0"]["command"].split()
+        if "--pipeline-parallel-size" not in cmd:
+            continue          # a block written by an earlier version of the generator
+        tp = int(cmd[cmd.index("--tensor-parallel-size") + 1])
+        pp = int(cmd[cmd.index("--pipeline-parallel-size") + 1])
+        model_path = cmd[cmd.index("--model") + 1]
+        k = cmd.index("--served-model-name")
+        model_name, extra = cmd[k + 1], " ".join(cmd[k + 2:])
+        name = want["vllm_0"]["container_name"].rsplit("_", 1)[0]
+        hf_dir = want["vllm_0"]["volumes"][0].split(":")[0]
+        conf = want["nginx"]["volumes"][0].split(":")[0] if "nginx" in want else None
+        got = yaml.safe_load(deploy.to_yaml(deploy.compose(n, tp, pp, name, model_path, model_name, hf_dir,
+                                                           nginx_conf_path=conf, extra_args=extra)))["services"]
+        assert list(got) == list(want), f.name
+        for i in range(n):
+            g, w = got[f"vllm_{i}"], want[f"vllm_{i}"]
+            for key in ("container_name", "ports", "shm_size", "ipc", "healthcheck"):
+                assert g[key] == w[key], (f.name, key)
+            assert g["command"].split() == w["command"].split(), f.name
+            ids = w["deploy"]["resources"]["reservations"]["devices"][0]["device_ids"]
+            assert f"HIP_VISIBLE_DEVICES={','.join(str(x) for x in ids)}" in g["environment"], f.name
+        if "nginx" in want:
+            assert got["nginx"] == want["nginx"], f.name
+        for key in ("container_name", "volumes", "entrypoint", "command", "profiles"):
+            assert got["benchmark"][key] == want["benchmark"][key], (f.name, key)
+        checked += 1
+    print(f"[deploy] {checked} recorded stacks regenerated")
+    assert checked >= 10
+
+
 def test_gpu_count_and_nginx_conf(deploy):
     text = "\n".join(["Agent 1", "  Device Type:             CPU", "Agent 2", "  Device Type:             GPU",
                       "  Compute Unit:            256", "Agent 3", "  Device Type:             GPU"])
