@@ -1,7 +1,8 @@
 // C ABI of libawq_mi355x.so: host-side validation and launch of the gfx950 kernels.
 // Every entry point checks its arguments before touching the device, launches on the
 // caller's stream and returns; nothing here allocates, synchronises or keeps state apart
-// from the thread-local last HIP error and the development variant switch.
+// from the thread-local last HIP error, the one-time kernel attribute set-up and the
+// development variant switch.  Launch shapes assume the MI355X's 256 CUs in 8 XCDs.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
