@@ -67,11 +67,11 @@ def main():
     ap.add_argument("--detail", action="store_true", help="per-point timings on stderr")
     ap.add_argument("--sweep-only", action="store_true",
                     help="only the timed decode sweep (no per-point, prefill, dequantize, MoE or CPU legs)")
-    ap.add_argument("--pmc-target", choices=("decode", "prefill"), default=None,
+    ap.add_argument("--pmc-target", choices=("decode", "prefill", "moe"), default=None,
                     help="counter-collection mode for rocprofv3 --pmc, no timing.  decode: the 16-launch "
                          "decode sweep twice (direct launches) plus four 256 MiB device copies "
                          "(calibration of FETCH_SIZE / WRITE_SIZE).  prefill: awq_gemm at o_proj, "
-                         "M=8192, three times")
+                         "M=8192, three times.  moe: the Qwen3-30B-A3B MoE block at T=512, five times")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -142,6 +142,18 @@ def main():
         torch.cuda.synchronize()
         log(f"[bench] pmc target: 3 x awq_gemm {name} M=8192 K={K} N={N} "
             f"({workloads.linear_flops(8192, K, N)} flops each)")
+        return
+    if args.pmc_target == "moe":
+        mq = workloads.QWEN3_MOE
+        H, E, topk, I = mq["hidden"], mq["experts"], mq["topk"], mq["inter"]
+        w13 = tuple(torch.stack(t) for t in zip(*[make_weights(H, 2 * I, G, dev, gen) for _ in range(E)]))
+        w2 = tuple(torch.stack(t) for t in zip(*[make_weights(I, H, G, dev, gen) for _ in range(E)]))
+        xm = torch.randn((512, H), device=dev, generator=gen).to(torch.float16)
+        lg = torch.randn((512, E), device=dev, generator=gen)
+        for _ in range(5):
+            sba.fused_moe_awq(xm, w13, w2, lg, topk, True)
+        torch.cuda.synchronize()
+        log(f"[bench] pmc target: 5 x MoE block, T=512, {E} experts, top-{topk}, hidden {H}, inter {I}")
         return
     if args.pmc_target == "decode":
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
