@@ -595,8 +595,10 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   p.nblk = nblk;
   p.ldy = fuse_act ? N / 2 : N;
   const int variant = g_gemv_variant.load(std::memory_order_relaxed);
-  // group blocks by XCD once experts average two blocks or more
-  p.grp = (long long)n_slots >= 2LL * tile_m * E ? 8 : 1;
+  // group blocks by XCD once most experts have a full block: runs of 8 from 0.75 blocks per
+  // expert on, runs of 32 from 1.5 (measured on 128 experts: 6 % at one block per expert, 15 %
+  // at 1.5, 3 - 4 % at 2 - 4 against runs of 8 or none; below 0.75 the order makes no difference)
+  p.grp = (long long)n_slots * 2 >= 3LL * tile_m * E ? 32 : ((long long)n_slots * 4 >= 3LL * tile_m * E ? 8 : 1);
   if (variant >= 0 && ((variant >> 2) & 7)) p.grp = 1 << (((variant >> 2) & 7) - 1);
   // few chunks of K and no split across workgroups: two column blocks per workgroup, two
   // waves each (three chunks per wave at K = 768 instead of 2 / 2 / 1 / 1)

@@ -55,7 +55,7 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 // ONE XCD, so the blocks that share an expert read its weights through the same L2 at about
 // the same time instead of fetching them once per XCD.  grp = 1 is the plain order (column
 // block fastest), used when few experts get more than one block.
-constexpr int MOE_BLOCK_GROUP_MAX = 16;
+constexpr int MOE_BLOCK_GROUP_MAX = 32;
 
 // 8-byte device-coherent store / load (relaxed, agent scope)
 __device__ __forceinline__ void st_coherent(float* p, f2 v) {
