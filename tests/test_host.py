@@ -63,6 +63,13 @@ def test_validation_happens_before_any_launch(lib):
                                   0, 0, 0, 0) == 4
     assert lib.awqmi_moe_gemm_f16(fake, fake, fake, fake, fake, fake, fake, fake, 0, 8, 2, 24, 4, 128, 64, 128,
                                   0, 0, 0, 0) == 7
+    # block rows of the MFMA form: 64 / 128 / 256 are accepted (so a bad group size is what is
+    # reported), 48 or 512 are not; the query sizes only the counters for them
+    for tile, want in ((64, 4), (128, 4), (256, 4), (48, 7), (512, 7)):
+        assert lib.awqmi_moe_gemm_f16(fake, fake, fake, fake, fake, fake, fake, fake, 0, 8, 2, tile, 4, 100, 64,
+                                      50, 0, 0, 0, 0) == want
+    assert lib.awqmi_moe_gemm_workspace_bytes(4096, 8, 1024, 1024, 0, 128) == 65536
+    assert lib.awqmi_moe_gemm_workspace_bytes(4096, 8, 1024, 1024, 0, 48) == 0
     assert lib.awqmi_silu_and_mul_f16(fake, fake, 4, 12, 0) == 1
     assert lib.awqmi_moe_sum_f16(fake, fake, 4, 2, 12, 0) == 1
     # whole-block MoE call: null operand, top-k beyond E, short workspace
