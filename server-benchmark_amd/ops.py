@@ -259,6 +259,8 @@ def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Ten
     _need(hidden_states, "hidden_states", torch.float16, 2)
     T, H = hidden_states.shape
     E = w13[0].shape[0]
+    if T == 0:
+        return hidden_states.new_empty((0, H))
     plain_routing = (scoring_func == "softmax" and e_score_correction_bias is None
                      and routed_scaling_factor == 1.0)
     if block_size is None and plain_routing:

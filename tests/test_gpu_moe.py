@@ -302,3 +302,15 @@ def test_moe_block_sigmoid_routing(sba, gpu):
     ref = awq_ref.moe_forward(c.x.numpy(), tuple(a.numpy() for a in c.w13), tuple(a.numpy() for a in c.w2),
                               ids, tw, 128)
     assert awq_ref.rel_frobenius(y, ref) <= TOL
+
+
+def test_empty_batches(sba, gpu):
+    """No tokens: every operator returns an empty result of the right shape and launches nothing."""
+    c = sba.workloads.make_moe_case(4, 256, 8, 2, 128, 128, seed=1).to(gpu)
+    y = sba.fused_moe_awq(c.x[:0], c.w13, c.w2, c.logits[:0], 2, True)
+    assert tuple(y.shape) == (0, 256) and y.dtype == torch.float16
+    y = sba.fused_moe_awq(c.x[:0], c.w13, c.w2, c.logits[:0], 2, True, block_size=16)
+    assert tuple(y.shape) == (0, 256)
+    lin = sba.workloads.make_linear_case(2, 256, 64, 128, seed=0).to(gpu)
+    y = sba.awq_gemm(lin.x[:0], lin.qweight, lin.scales, lin.qzeros, 0)
+    assert tuple(y.shape) == (0, 64) and y.dtype == torch.float16
