@@ -153,6 +153,7 @@ static int ensure_kernel_attributes() {
   }
   const void* align[] = {
       reinterpret_cast<const void*>(moe_align_kernel),
+      reinterpret_cast<const void*>(moe_align_count_kernel), reinterpret_cast<const void*>(moe_align_place_kernel),
       reinterpret_cast<const void*>(moe_route_align_kernel<1, false>), reinterpret_cast<const void*>(moe_route_align_kernel<2, false>),
       reinterpret_cast<const void*>(moe_route_align_kernel<4, false>), reinterpret_cast<const void*>(moe_route_align_kernel<8, false>),
       reinterpret_cast<const void*>(moe_route_align_kernel<16, false>)};
@@ -653,6 +654,9 @@ int awqmi_moe_sum_f16(const void* in, void* out, int T, int topk, int H, void* s
 }
 
 namespace {
+constexpr int MOE_ALIGN_PARTS_MAX = 64;      // workgroups of the multi-workgroup align
+constexpr int MOE_ALIGN_SPLIT_MIN = 16384;   // slots from which it is used (4096 per workgroup)
+
 // Rows per block for the two expert GEMMs of one MoE block: 16 (the skinny kernel) or 64 /
 // 128 / 256 (the MFMA kernel's expert-grouped form).  Cost model fitted on measurements over
 // three expert shapes (2048/768 x 128 experts, 6144/2560 x 160, 4096/14336 x 8):
@@ -695,6 +699,7 @@ struct FusedMoeLayout {
   size_t gemm_ws, ids, wts, sorted, experts, npp, h13, act, o, total;
   size_t gemm_ws_bytes;
   int n_slots, cap, tile;
+  size_t tab;      // per-part expert counts / first positions of the multi-workgroup align
 };
 FusedMoeLayout fused_moe_layout(int T, int H, int inter, int E, int topk, int tile) {
   FusedMoeLayout L{};
@@ -712,6 +717,7 @@ FusedMoeLayout fused_moe_layout(int T, int H, int inter, int E, int topk, int ti
   L.sorted = off;  off += up((size_t)L.cap * 4);
   L.experts = off; off += up((size_t)(L.cap / L.tile) * 4);
   L.npp = off;     off += 256;
+  L.tab = off;     off += up((size_t)MOE_ALIGN_PARTS_MAX * E * 4);
   L.h13 = off;     off += up((size_t)L.n_slots * 2 * inter * 2);
   L.act = off;     off += up((size_t)L.n_slots * inter * 2);
   L.o = off;       off += up((size_t)L.n_slots * H * 2);
@@ -765,7 +771,26 @@ int awqmi_fused_moe_f16(const void* hidden, const float* router_logits, const in
   } else {
     st = awqmi_moe_topk_softmax_f32(router_logits, T, E, topk, renormalize, ids, wts, stream);
     if (st) return st;
-    st = awqmi_moe_align(ids, L.n_slots, E, tile, sorted, experts, npp, stream);
+    const int valign = g_gemv_variant.load(std::memory_order_relaxed);
+    if (L.n_slots >= MOE_ALIGN_SPLIT_MIN && !(valign >= 0 && (valign & 16384))) {
+      // long slot lists: count per part, scan, place per part (three launches, many workgroups)
+      if (int s2 = ensure_kernel_attributes()) return s2;
+      int parts = (L.n_slots + 4095) / 4096;
+      if (parts > MOE_ALIGN_PARTS_MAX) parts = MOE_ALIGN_PARTS_MAX;
+      const int part = ((L.n_slots + parts - 1) / parts + 63) / 64 * 64;
+      parts = (L.n_slots + part - 1) / part;
+      int32_t* tab = reinterpret_cast<int32_t*>(ws + L.tab);
+      const size_t lds = (size_t)(MOE_ALIGN_WAVES + 2) * E * sizeof(int);
+      hipStream_t hs = (hipStream_t)stream;
+      hipLaunchKernelGGL(moe_align_count_kernel, dim3(parts), dim3(1024), lds, hs, ids, L.n_slots, E, part, tab);
+      hipLaunchKernelGGL(moe_align_scan_kernel, dim3(1), dim3(1024), (size_t)2 * E * sizeof(int), hs, L.n_slots, E,
+                         tile, L.cap, parts, tab, sorted, experts, npp);
+      hipLaunchKernelGGL(moe_align_place_kernel, dim3(parts), dim3(1024), lds, hs, ids, L.n_slots, E, part, tab,
+                         sorted);
+      st = launch_status();
+    } else {
+      st = awqmi_moe_align(ids, L.n_slots, E, tile, sorted, experts, npp, stream);
+    }
     if (st) return st;
   }
   const int Gn = norm_group(H, group);

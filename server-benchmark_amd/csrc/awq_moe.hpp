@@ -123,22 +123,30 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__
 // position per (wave, expert) lives in LDS and is bumped by one LDS atomic per slot after all
 // lanes of the batch have read it.
 constexpr int MOE_ALIGN_WAVES = 16;
+// MODE 0: the whole job in one workgroup.  For long slot lists the job is split over the
+// workgroups of three launches (one workgroup scatters about one slot per clock, whatever it
+// does): MODE 1 = count the experts of this workgroup's part [s0, s1) into block_cnt[block][E];
+// (moe_align_scan_kernel turns the counts into each part's first position per expert and writes
+// the padding;) MODE 2 = place this part's slots from block_start[block][E].
+template <int MODE>
 __device__ __forceinline__ void moe_align_block(const int* __restrict__ ids, int n, int E, int tile_m,
                                                 int cap, int* __restrict__ sorted,
                                                 int* __restrict__ expert_ids, int* __restrict__ npp,
-                                                int* sm) {
+                                                int* sm, int s0 = 0, int s1 = 0,
+                                                int* __restrict__ block_tab = nullptr) {
   constexpr int NWV = MOE_ALIGN_WAVES;
   int* cnt = sm;               // [NWV][E], later the running write position
   int* padded = sm + NWV * E;  // [E]
   int* start = padded + E;     // [E]
   __shared__ int s_total;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  if (MODE == 0) { s0 = 0; s1 = n; }
 
   for (int i = tid; i < NWV * E; i += 1024) cnt[i] = 0;
   __syncthreads();
 
-  const int seg = ((n + NWV * 64 - 1) / (NWV * 64)) * 64;
-  const int sb = wave * seg, se = min(n, sb + seg);
+  const int seg = ((s1 - s0 + NWV * 64 - 1) / (NWV * 64)) * 64;
+  const int sb = s0 + wave * seg, se = min(s1, sb + seg);
   // ids are read eight batches of 64 at a time (eight loads in flight instead of one
   // dependent load per batch); the first eight batches stay in registers for the second pass
   constexpr int NB = 8;
@@ -168,6 +176,22 @@ __device__ __forceinline__ void moe_align_block(const int* __restrict__ ids, int
   }
   __syncthreads();
 
+  if (MODE == 1) {
+    for (int e = tid; e < E; e += 1024) {
+      int tot = 0;
+      for (int w = 0; w < NWV; ++w) tot += cnt[w * E + e];
+      block_tab[(size_t)blockIdx.x * E + e] = tot;
+    }
+    return;
+  }
+  if (MODE == 2) {
+    for (int e = tid; e < E; e += 1024) {
+      int pos = block_tab[(size_t)blockIdx.x * E + e];
+      for (int w = 0; w < NWV; ++w) { const int c = cnt[w * E + e]; cnt[w * E + e] = pos; pos += c; }
+    }
+    __syncthreads();
+  }
+  if constexpr (MODE == 0) {
   for (int e = tid; e < E; e += 1024) {
     int tot = 0;
     for (int w = 0; w < NWV; ++w) tot += cnt[w * E + e];
@@ -198,14 +222,15 @@ __device__ __forceinline__ void moe_align_block(const int* __restrict__ ids, int
   const int total = s_total;
   for (int e = tid; e < E; e += 1024) {
     int pos = start[e];
-    const int s0 = pos;
+    const int e0 = pos;
     for (int w = 0; w < NWV; ++w) { const int c = cnt[w * E + e]; cnt[w * E + e] = pos; pos += c; }
-    for (int i = pos; i < s0 + padded[e]; ++i) sorted[i] = n;            // pad entries
-    for (int b = 0; b < padded[e] / tile_m; ++b) expert_ids[s0 / tile_m + b] = e;
+    for (int i = pos; i < e0 + padded[e]; ++i) sorted[i] = n;            // pad entries
+    for (int b = 0; b < padded[e] / tile_m; ++b) expert_ids[e0 / tile_m + b] = e;
   }
   for (int i = total + tid; i < cap; i += 1024) sorted[i] = n;           // unused tail
   for (int i = total / tile_m + tid; i < cap / tile_m; i += 1024) expert_ids[i] = -1;
   __syncthreads();
+  }   // MODE == 0
 
   const int nbits = 32 - __builtin_clz(max(E - 1, 1));
   auto place = [&](int i, int e) {
@@ -250,7 +275,98 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
                                                          int* __restrict__ expert_ids,
                                                          int* __restrict__ npp) {
   extern __shared__ int sm[];
-  moe_align_block(ids, n, E, tile_m, cap, sorted, expert_ids, npp, sm);
+  moe_align_block<0>(ids, n, E, tile_m, cap, sorted, expert_ids, npp, sm);
+}
+
+// Long slot lists: part b of gridDim.x parts covers slots [b * part, (b + 1) * part).
+__global__ __launch_bounds__(1024) void moe_align_count_kernel(const int* __restrict__ ids, int n, int E,
+                                                               int part, int* __restrict__ block_cnt) {
+  extern __shared__ int sm[];
+  const int s0 = min(n, (int)blockIdx.x * part), s1 = min(n, s0 + part);
+  moe_align_block<1>(ids, n, E, 1, 0, nullptr, nullptr, nullptr, sm, s0, s1, block_cnt);
+}
+
+// One workgroup: per expert the padded length and first position, then every part's first
+// position per expert (in place: counts in, positions out), the padding entries, the block
+// owners and the unused tails.
+__global__ __launch_bounds__(1024) void moe_align_scan_kernel(int n, int E, int tile_m, int cap, int parts,
+                                                              int* __restrict__ block_tab,
+                                                              int* __restrict__ sorted,
+                                                              int* __restrict__ expert_ids,
+                                                              int* __restrict__ npp) {
+  extern __shared__ int sm[];
+  int* padded = sm;        // [E]
+  int* start = sm + E;     // [E]
+  __shared__ int s_total;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // thread e keeps its expert's counts of all parts in registers (one memory round trip;
+  // E <= 1024 = the workgroup size, parts <= 64)
+  constexpr int PMAX = 64;
+  int c[PMAX];
+  const int my_e = tid < E ? tid : 0;
+#pragma unroll
+  for (int b = 0; b < PMAX; ++b) c[b] = block_tab[(size_t)min(b, parts - 1) * E + my_e];
+  if (tid < E) {
+    int tot = 0;
+#pragma unroll
+    for (int b = 0; b < PMAX; ++b) tot += b < parts ? c[b] : 0;
+    padded[tid] = (tot + tile_m - 1) / tile_m * tile_m;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    const int per = (E + 63) / 64;
+    int local = 0;
+    for (int k = 0; k < per; ++k) {
+      const int e = lane * per + k;
+      if (e < E) local += padded[e];
+    }
+    int incl = local;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int v = __shfl_up(incl, o);
+      if (lane >= o) incl += v;
+    }
+    int pos = incl - local;
+    for (int k = 0; k < per; ++k) {
+      const int e = lane * per + k;
+      if (e < E) { start[e] = pos; pos += padded[e]; }
+    }
+    if (lane == 63) { s_total = incl; npp[0] = incl; }
+  }
+  __syncthreads();
+  const int total = s_total;
+  if (tid < E) {
+    const int e = tid;
+    int pos = start[e];
+    const int e0 = pos;
+#pragma unroll
+    for (int b = 0; b < PMAX; ++b) {
+      if (b < parts) {
+        block_tab[(size_t)b * E + e] = pos;
+        pos += c[b];
+      }
+    }
+    padded[e] = pos;          // from here on: first padding position of the expert's run
+    (void)e0;
+  }
+  __syncthreads();
+  // padding entries and block owners, one wave per expert at a time (coalesced stores)
+  for (int e = wave; e < E; e += 16) {
+    const int e0 = start[e];
+    const int e1 = e + 1 < E ? start[e + 1] : total;
+    for (int i = padded[e] + lane; i < e1; i += 64) sorted[i] = n;
+    for (int b = e0 / tile_m + lane; b < e1 / tile_m; b += 64) expert_ids[b] = e;
+  }
+  for (int i = total + tid; i < cap; i += 1024) sorted[i] = n;
+  for (int i = total / tile_m + tid; i < cap / tile_m; i += 1024) expert_ids[i] = -1;
+}
+
+__global__ __launch_bounds__(1024) void moe_align_place_kernel(const int* __restrict__ ids, int n, int E,
+                                                               int part, int* __restrict__ block_start,
+                                                               int* __restrict__ sorted) {
+  extern __shared__ int sm[];
+  const int s0 = min(n, (int)blockIdx.x * part), s1 = min(n, s0 + part);
+  moe_align_block<2>(ids, n, E, 1, 0, sorted, nullptr, nullptr, sm, s0, s1, block_start);
 }
 
 // Routing and align in one launch for batches of at most 16 tokens (one wave per token, the
@@ -268,7 +384,7 @@ __global__ __launch_bounds__(1024) void moe_route_align_kernel(const float* __re
   const int wave = threadIdx.x >> 6;
   if (wave < T) moe_topk_token<PER, SIGMOID>(logits, bias, wave, E, topk, renorm, scale, ids, wts);
   __syncthreads();   // the ids written above are read back by the same workgroup
-  moe_align_block(ids, T * topk, E, tile_m, cap, sorted, expert_ids, npp, sm);
+  moe_align_block<0>(ids, T * topk, E, tile_m, cap, sorted, expert_ids, npp, sm);
 }
 
 __global__ __launch_bounds__(256) void silu_and_mul_kernel(const half_t* __restrict__ in,

@@ -314,3 +314,19 @@ def test_empty_batches(sba, gpu):
     lin = sba.workloads.make_linear_case(2, 256, 64, 128, seed=0).to(gpu)
     y = sba.awq_gemm(lin.x[:0], lin.qweight, lin.scales, lin.qzeros, 0)
     assert tuple(y.shape) == (0, 64) and y.dtype == torch.float16
+
+
+@pytest.mark.parametrize("T,E,topk", [(2048, 128, 8), (2500, 60, 7), (20000, 8, 2)])
+def test_fused_call_with_long_slot_lists(sba, gpu, T, E, topk):
+    """From 16384 slots on the one-call path sorts the slots with several workgroups (count,
+    scan, place); its result must equal the step-by-step path, whose align is the single
+    workgroup checked against the oracle above."""
+    H, I = 256, 128
+    c = sba.workloads.make_moe_case(T, H, E, topk, I, 128, seed=T + E).to(gpu)
+    assert T * topk >= 16384
+    one = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True)
+    from server_benchmark_amd import _lib
+    bs = _lib.load().awqmi_fused_moe_block_rows(T, H, I, E, topk, 128)
+    step = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True, block_size=bs)
+    assert torch.equal(one, step)
+    assert torch.equal(one, sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True))
