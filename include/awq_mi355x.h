@@ -168,6 +168,18 @@ int awqmi_fused_moe_f16(const void* hidden_f16, const float* router_logits, cons
                         void* out_f16, int T, int H, int inter, int E, int topk, int group,
                         int renormalize, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same block with the routing of awqmi_moe_topk_f32: scoring 0 = softmax, 1 = sigmoid with an
+ * optional score-correction bias fp32 [E] in the selection key (NULL for none; not allowed with
+ * softmax), weights optionally renormalised and multiplied by routed_scale.  Stands in for the
+ * same AWQMoEMethod.apply with scoring_func / e_score_correction_bias / routed_scaling_factor
+ * set (the sigmoid-routed MoE checkpoints of reference config.yaml:51).  Workspace as above. */
+int awqmi_fused_moe_routed_f16(const void* hidden_f16, const float* router_logits, const float* score_bias,
+                               const int32_t* w13_qweight, const void* w13_scales_f16,
+                               const int32_t* w13_qzeros, const int32_t* w2_qweight,
+                               const void* w2_scales_f16, const int32_t* w2_qzeros, void* out_f16, int T,
+                               int H, int inter, int E, int topk, int group, int scoring, int renormalize,
+                               float routed_scale, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Development hook: choose among equivalent kernel variants of the skinny GEMM
  * (-1 = library default).  Returns the previous value.  Not part of the stable surface. */
 int awqmi_set_gemv_variant(int variant);

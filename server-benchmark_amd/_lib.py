@@ -37,6 +37,9 @@ SIGNATURES = {
     "awqmi_fused_moe_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t,
                                     c_void_p]),
+    "awqmi_fused_moe_routed_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                           c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                           c_int, c_int, ctypes.c_float, c_void_p, c_size_t, c_void_p]),
     "awqmi_set_gemv_variant": (c_int, [c_int]),
 }
 

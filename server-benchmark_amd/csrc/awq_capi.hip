@@ -745,12 +745,23 @@ int awqmi_fused_moe_f16(const void* hidden, const float* router_logits, const in
                         const int32_t* w2_z, void* out, int T, int H, int inter, int E, int topk,
                         int group, int renormalize, void* workspace, size_t workspace_bytes,
                         void* stream) {
+  return awqmi_fused_moe_routed_f16(hidden, router_logits, nullptr, w13_q, w13_s, w13_z, w2_q, w2_s, w2_z, out, T,
+                                    H, inter, E, topk, group, 0, renormalize, 1.f, workspace, workspace_bytes,
+                                    stream);
+}
+
+int awqmi_fused_moe_routed_f16(const void* hidden, const float* router_logits, const float* score_bias,
+                               const int32_t* w13_q, const void* w13_s, const int32_t* w13_z,
+                               const int32_t* w2_q, const void* w2_s, const int32_t* w2_z, void* out, int T,
+                               int H, int inter, int E, int topk, int group, int scoring, int renormalize,
+                               float routed_scale, void* workspace, size_t workspace_bytes, void* stream) {
   if (!hidden || !router_logits || !w13_q || !w13_s || !w13_z || !w2_q || !w2_s || !w2_z || !out ||
       !workspace)
     return AWQMI_NULL_POINTER;
   if (T <= 0 || H <= 0 || inter <= 0 || E <= 0 || H % 8 != 0 || inter % 8 != 0) return AWQMI_BAD_SHAPE;
   if (topk <= 0 || topk > E || topk > 64 || E > AWQMI_MAX_EXPERTS || (long long)T * topk > (1LL << 30))
     return AWQMI_BAD_ARGUMENT;
+  if ((scoring != 0 && scoring != 1) || (scoring == 0 && score_bias)) return AWQMI_BAD_ARGUMENT;
   if (!aligned16(workspace)) return AWQMI_BAD_ALIGN;
   const int tile = moe_pick_tile(T * topk, E, H, inter, group);
   const FusedMoeLayout L = fused_moe_layout(T, H, inter, E, topk, tile);
@@ -765,11 +776,13 @@ int awqmi_fused_moe_f16(const void* hidden, const float* router_logits, const in
   void* act = ws + L.act;
   void* o = ws + L.o;
   int st;
-  if (T <= MOE_ALIGN_WAVES) {
+  const bool plain_routing = scoring == 0 && !score_bias && routed_scale == 1.f;
+  if (T <= MOE_ALIGN_WAVES && plain_routing) {
     st = moe_route_align_small(router_logits, T, E, topk, renormalize, ids, wts, tile, sorted, experts, npp, stream);
     if (st) return st;
   } else {
-    st = awqmi_moe_topk_softmax_f32(router_logits, T, E, topk, renormalize, ids, wts, stream);
+    st = awqmi_moe_topk_f32(router_logits, score_bias, T, E, topk, scoring, renormalize, routed_scale, ids, wts,
+                            stream);
     if (st) return st;
     const int valign = g_gemv_variant.load(std::memory_order_relaxed);
     if (L.n_slots >= MOE_ALIGN_SPLIT_MIN && !(valign >= 0 && (valign & 16384))) {

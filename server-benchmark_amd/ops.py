@@ -254,16 +254,17 @@ def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Ten
     """One AWQ MoE block: route -> align -> grouped GEMM (w13) -> SiLU*up -> grouped GEMM (w2,
     scaled by the routing weight) -> sum over slots.  w13 / w2 are (qweight, scales, qzeros)
     with a leading expert dimension; w13 columns are [gate | up].  With block_size left at
-    None and plain softmax routing the block runs as one library call; a block size, sigmoid
-    scoring, a score-correction bias or a routed scaling factor select the step-by-step path."""
+    None the block runs as one library call (softmax routing, or sigmoid scoring with an
+    optional score-correction bias; routing weights times routed_scaling_factor); a block size
+    selects the step-by-step path over blocks of that size."""
     _need(hidden_states, "hidden_states", torch.float16, 2)
     T, H = hidden_states.shape
     E = w13[0].shape[0]
     if T == 0:
         return hidden_states.new_empty((0, H))
-    plain_routing = (scoring_func == "softmax" and e_score_correction_bias is None
-                     and routed_scaling_factor == 1.0)
-    if block_size is None and plain_routing:
+    if scoring_func not in ("softmax", "sigmoid"):
+        raise ValueError(f"scoring_func must be 'softmax' or 'sigmoid', got {scoring_func!r}")
+    if block_size is None:
         # the whole block in one library call, intermediates in the workspace
         for i, (t, dt) in enumerate(zip(tuple(w13) + tuple(w2), (torch.int32, torch.float16, torch.int32) * 2)):
             _need(t, f"w13/w2[{i}]", dt, 3)
@@ -278,14 +279,27 @@ def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Ten
         _need(lg, "gating_output", torch.float32, 2)
         if tuple(lg.shape) != (T, E):
             raise ValueError(f"gating_output shape {tuple(lg.shape)} != ({T}, {E})")
+        bias = 0
+        if e_score_correction_bias is not None:
+            if scoring_func != "sigmoid":
+                raise ValueError("e_score_correction_bias belongs to sigmoid scoring")
+            bias_t = e_score_correction_bias
+            if bias_t.dtype != torch.float32 or not bias_t.is_contiguous():
+                bias_t = bias_t.float().contiguous()
+            _need(bias_t, "e_score_correction_bias", torch.float32, 1)
+            if bias_t.numel() != E:
+                raise ValueError(f"e_score_correction_bias has {bias_t.numel()} entries for {E} experts")
+            bias = bias_t.data_ptr()
         lib = _lib.load()
         nbytes = lib.awqmi_fused_moe_workspace_bytes(T, H, inter, E, topk)
         ws = get_workspace(hidden_states.device, nbytes)
         out = torch.empty((T, H), dtype=torch.float16, device=hidden_states.device)
-        st = lib.awqmi_fused_moe_f16(hidden_states.data_ptr(), lg.data_ptr(), w13[0].data_ptr(), w13[1].data_ptr(),
-                                     w13[2].data_ptr(), w2[0].data_ptr(), w2[1].data_ptr(), w2[2].data_ptr(),
-                                     out.data_ptr(), T, H, inter, E, topk, G1, int(renormalize), ws.data_ptr(),
-                                     ws.numel(), _stream_ptr(hidden_states.device))
+        st = lib.awqmi_fused_moe_routed_f16(hidden_states.data_ptr(), lg.data_ptr(), bias, w13[0].data_ptr(),
+                                            w13[1].data_ptr(), w13[2].data_ptr(), w2[0].data_ptr(),
+                                            w2[1].data_ptr(), w2[2].data_ptr(), out.data_ptr(), T, H, inter, E,
+                                            topk, G1, 1 if scoring_func == "sigmoid" else 0, int(renormalize),
+                                            float(routed_scaling_factor), ws.data_ptr(), ws.numel(),
+                                            _stream_ptr(hidden_states.device))
         _lib.check(st, "fused_moe_awq")
         return out
     T = hidden_states.shape[0]

@@ -302,6 +302,36 @@ def test_moe_block_sigmoid_routing(sba, gpu):
     ref = awq_ref.moe_forward(c.x.numpy(), tuple(a.numpy() for a in c.w13), tuple(a.numpy() for a in c.w2),
                               ids, tw, 128)
     assert awq_ref.rel_frobenius(y, ref) <= TOL
+    # the one-call path above and the step-by-step path run the same kernels on the same routing
+    step = sba.fused_moe_awq(cg.x, cg.w13, cg.w2, cg.logits, 4, True, scoring_func="sigmoid",
+                             e_score_correction_bias=bias.to(gpu), routed_scaling_factor=1.5, block_size=16)
+    assert np.array_equal(step.cpu().numpy(), y)
+
+
+@pytest.mark.parametrize("T", [64, 3000])
+def test_moe_block_sigmoid_routing_larger_batches(sba, gpu, T):
+    """Sigmoid-routed block at batch sizes that take the separate routing kernel and, at 3000
+    tokens, the multi-workgroup align and the MFMA blocks: against the dense expert path with the
+    routing kernel's own ids and weights."""
+    H, E, topk, I = 512, 32, 6, 256
+    c = sba.workloads.make_moe_case(T, H, E, topk, I, 128, seed=T).to(gpu)
+    bias = (torch.randn((E,), generator=torch.Generator().manual_seed(9)) * 0.1).to(gpu)
+    y = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True, scoring_func="sigmoid",
+                          e_score_correction_bias=bias, routed_scaling_factor=2.5)
+    w, ids = sba.topk_route(c.logits, topk, True, "sigmoid", bias, 2.5)
+    ref = torch.zeros((T, H), dtype=torch.float32, device=gpu)
+    for e in range(E):
+        tok, slot = torch.nonzero(ids == e, as_tuple=True)
+        if tok.numel() == 0:
+            continue
+        W13 = sba.awq_dequantize(c.w13[0][e], c.w13[1][e], c.w13[2][e]).float()
+        W2 = sba.awq_dequantize(c.w2[0][e], c.w2[1][e], c.w2[2][e]).float()
+        h = (c.x[tok].float() @ W13).half().float()
+        a = (torch.nn.functional.silu(h[:, :I]) * h[:, I:]).half().float()
+        ref.index_add_(0, tok, ((a @ W2) * w[tok, slot][:, None]).half().float())
+    err = float((y.float() - ref).norm() / ref.norm())
+    print(f"[moe sigmoid T={T}] rel_fro={err:.2e}", flush=True)
+    assert err <= TOL
 
 
 def test_empty_batches(sba, gpu):

@@ -77,6 +77,12 @@ def test_validation_happens_before_any_launch(lib):
     assert lib.awqmi_fused_moe_f16(*ok[:8], 0, 4, 256, 128, 8, 2, 128, 1, fake, 1 << 30, 0) == 6
     assert lib.awqmi_fused_moe_f16(*ok, 4, 256, 128, 8, 9, 128, 1, fake, 1 << 30, 0) == 7
     assert lib.awqmi_fused_moe_f16(*ok, 4, 256, 128, 8, 2, 128, 1, fake, 1024, 0) == 3
+    # routed form: a bias with softmax scoring, an unknown scoring id
+    okr = [fake, fake, fake] + [fake] * 7
+    assert lib.awqmi_fused_moe_routed_f16(*okr, 4, 256, 128, 8, 2, 128, 0, 1, 1.0, fake, 1 << 30, 0) == 7
+    okr[2] = 0
+    assert lib.awqmi_fused_moe_routed_f16(*okr, 4, 256, 128, 8, 2, 128, 2, 1, 1.0, fake, 1 << 30, 0) == 7
+    assert lib.awqmi_fused_moe_routed_f16(*okr, 4, 256, 128, 8, 2, 128, 1, 1, 2.5, fake, 1024, 0) == 3
     assert lib.awqmi_fused_moe_f16(*ok, 4, 250, 128, 8, 2, 128, 1, fake, 1 << 30, 0) == 1
 
 
