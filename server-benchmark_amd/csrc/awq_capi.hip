@@ -171,7 +171,7 @@ template <int P>
 static int moe_route_align_launch(const float* logits, int T, int E, int topk, int renormalize,
                                   int32_t* ids, float* wts, int tile_m, int cap, int32_t* sorted,
                                   int32_t* experts, int32_t* npp, hipStream_t st) {
-  if (int st = ensure_kernel_attributes()) return st;
+  if (const int rc = ensure_kernel_attributes()) return rc;
   hipLaunchKernelGGL((moe_route_align_kernel<P, false>), dim3(1), dim3(1024),
                      (size_t)(MOE_ALIGN_WAVES + 2) * E * sizeof(int), st, logits, (const float*)nullptr, T, E,
                      topk, renormalize, 1.f, ids, wts, tile_m, cap, sorted, experts, npp);
@@ -218,7 +218,7 @@ int awqmi_dequantize_f16(const int32_t* qweight, const void* scales, const int32
                          void* out, int K, int N, int group, void* stream) {
   if (!qweight || !scales || !qzeros || !out) return AWQMI_NULL_POINTER;
   const int G = norm_group(K, group);
-  if (int st = check_awq_shape(K, N, G)) return st;
+  if (const int rc = check_awq_shape(K, N, G)) return rc;
   if (!aligned16(scales) || !aligned16(out) || !aligned16(qweight) || !aligned16(qzeros))
     return AWQMI_BAD_ALIGN;
   const int NW = N / 8;
@@ -229,13 +229,16 @@ int awqmi_dequantize_f16(const int32_t* qweight, const void* scales, const int32
   half_t* o = reinterpret_cast<half_t*>(out);
   const unsigned gx = (NW + 255) / 256;
 #define AWQMI_DQ(R)                                                                              \
-  hipLaunchKernelGGL((awq_dequant_kernel<R>), dim3(gx, K / R), dim3(256), 0, st, qw, sc, qz, o, K, \
-                     NW, G)
-  if (G % 16 == 0) AWQMI_DQ(16);
-  else if (G % 8 == 0) AWQMI_DQ(8);
-  else if (G % 4 == 0) AWQMI_DQ(4);
-  else if (G % 2 == 0) AWQMI_DQ(2);
-  else AWQMI_DQ(1);
+  for (int k0 = 0; k0 < K; k0 += 65535 * R) {                                                    \
+    const int slabs = (K - k0) / R < 65535 ? (K - k0) / R : 65535;                               \
+    hipLaunchKernelGGL((awq_dequant_kernel<R>), dim3(gx, slabs), dim3(256), 0, st, qw, sc, qz, o, k0, \
+                       NW, G);                                                                   \
+  }
+  if (G % 16 == 0) AWQMI_DQ(16)
+  else if (G % 8 == 0) AWQMI_DQ(8)
+  else if (G % 4 == 0) AWQMI_DQ(4)
+  else if (G % 2 == 0) AWQMI_DQ(2)
+  else AWQMI_DQ(1)
 #undef AWQMI_DQ
   return launch_status();
 }
@@ -274,7 +277,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
                    int split_k, void* stream) {
   if (!x || !qweight || !scales || !qzeros || !y) return AWQMI_NULL_POINTER;
   const int G = norm_group(K, group);
-  if (int st = check_awq_shape(K, N, G)) return st;
+  if (const int rc = check_awq_shape(K, N, G)) return rc;
   if (M <= 0) return AWQMI_BAD_SHAPE;
   if (split_k < 0 || split_k > AWQMI_MAX_SPLIT_K) return AWQMI_BAD_ARGUMENT;
   if (!aligned16(x) || !aligned16(scales) || !aligned16(qweight) || !aligned16(qzeros) ||
@@ -329,30 +332,30 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   // 32-bit, so every operand must stay below 4 GiB
   const bool pow2g = (G & (G - 1)) == 0 && G >= 8;
   if (mfma_ok) {
-    if (int st = ensure_kernel_attributes()) return st;
+    if (const int rc = ensure_kernel_attributes()) return rc;
     const int slab = mfma_slab_rows(M, K);
     for (int r0 = 0; r0 < M; r0 += slab) {
-    const int Ms = M - r0 < slab ? M - r0 : slab;
-    MfmaGemmParams p{};
-    p.x = xx + (size_t)r0 * K; p.qw = qw; p.sc = sc; p.qz = qz; p.y = yy + (size_t)r0 * N;
-    p.M = Ms; p.K = K; p.N = N; p.NW = NW; p.G = G;
-    p.gshift = 0;
-    if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
-    // at most 64 / 128 / 192 rows: one row of smaller tiles instead of a padded 256-row tile
-    const int mi = Ms <= 64 ? 1 : (Ms <= 128 ? 2 : (Ms <= 192 ? 3 : 4));
-    p.mt = mi < 4 ? 1 : (Ms + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
-    p.total = p.mt * p.nt;
-    MfmaPlan pl = plan_mfma(Ms, K, N);
-    // the K split needs the caller's workspace (counters + partial tiles); without it every
-    // tile runs on one workgroup
-    if (pl.sk_tiles > 0 && (!workspace || !aligned16(workspace) ||
-                            workspace_bytes < AWQMI_WS_COUNTER_BYTES + pl.part_bytes))
-      pl = MfmaPlan{p.total, 0, 1, 0};
-    p.dp_tiles = pl.dp_tiles; p.sk_tiles = pl.sk_tiles; p.sk_split = pl.sk_split;
-    p.per_xcd = (pl.dp_tiles + 7) / 8;
-    p.sk_part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
-                          : nullptr;
-    const dim3 grid(p.per_xcd * 8 + p.sk_tiles * p.sk_split);
+      const int Ms = M - r0 < slab ? M - r0 : slab;
+      MfmaGemmParams p{};
+      p.x = xx + (size_t)r0 * K; p.qw = qw; p.sc = sc; p.qz = qz; p.y = yy + (size_t)r0 * N;
+      p.M = Ms; p.K = K; p.N = N; p.NW = NW; p.G = G;
+      p.gshift = 0;
+      if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
+      // at most 64 / 128 / 192 rows: one row of smaller tiles instead of a padded 256-row tile
+      const int mi = Ms <= 64 ? 1 : (Ms <= 128 ? 2 : (Ms <= 192 ? 3 : 4));
+      p.mt = mi < 4 ? 1 : (Ms + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
+      p.total = p.mt * p.nt;
+      MfmaPlan pl = plan_mfma(Ms, K, N);
+      // the K split needs the caller's workspace (counters + partial tiles); without it every
+      // tile runs on one workgroup
+      if (pl.sk_tiles > 0 && (!workspace || !aligned16(workspace) ||
+                              workspace_bytes < AWQMI_WS_COUNTER_BYTES + pl.part_bytes))
+        pl = MfmaPlan{p.total, 0, 1, 0};
+      p.dp_tiles = pl.dp_tiles; p.sk_tiles = pl.sk_tiles; p.sk_split = pl.sk_split;
+      p.per_xcd = (pl.dp_tiles + 7) / 8;
+      p.sk_part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
+                            : nullptr;
+      const dim3 grid(p.per_xcd * 8 + p.sk_tiles * p.sk_split);
 #define AWQMI_MFMA(MIV, NWVV)                                                                      \
   do {                                                                                           \
     if (pow2g)                                                                                   \
@@ -363,21 +366,26 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
       hipLaunchKernelGGL((awq_gemm_mfma_reduce_kernel<MIV, NWVV>), dim3(p.sk_tiles * MIV * (16 / NWVV)),       \
                          dim3(64 * NWVV), 0, st, p);                                              \
   } while (0)
-    const bool eight = !(g_gemv_variant.load(std::memory_order_relaxed) >= 0 &&
-                         (g_gemv_variant.load(std::memory_order_relaxed) & 512));
-    if (mi == 1 && eight) AWQMI_MFMA(1, 8);
-    else if (mi == 2 && eight) AWQMI_MFMA(2, 8);
-    else if (mi == 1) AWQMI_MFMA(1, 4);
-    else if (mi == 2) AWQMI_MFMA(2, 4);
-    else if (mi == 3) AWQMI_MFMA(3, 4);
-    else AWQMI_MFMA(4, 4);
+      const bool eight = !(g_gemv_variant.load(std::memory_order_relaxed) >= 0 &&
+                           (g_gemv_variant.load(std::memory_order_relaxed) & 512));
+      if (mi == 1 && eight) AWQMI_MFMA(1, 8);
+      else if (mi == 2 && eight) AWQMI_MFMA(2, 8);
+      else if (mi == 1) AWQMI_MFMA(1, 4);
+      else if (mi == 2) AWQMI_MFMA(2, 4);
+      else if (mi == 3) AWQMI_MFMA(3, 4);
+      else AWQMI_MFMA(4, 4);
 #undef AWQMI_MFMA
     }
     return launch_status();
   }
 
-  hipLaunchKernelGGL(awq_gemm_generic_kernel, dim3((NW + 255) / 256, M), dim3(256), 0, st, xx, qw, sc,
-                     qz, yy, M, K, NW, G);
+  // any other shape: one thread per packed word and row; the row index is the grid's second
+  // dimension (at most 65535), so more rows run as consecutive slabs
+  for (int r0 = 0; r0 < M; r0 += 32768) {
+    const int Ms = M - r0 < 32768 ? M - r0 : 32768;
+    hipLaunchKernelGGL(awq_gemm_generic_kernel, dim3((NW + 255) / 256, Ms), dim3(256), 0, st,
+                       xx + (size_t)r0 * K, qw, sc, qz, yy + (size_t)r0 * N, Ms, K, NW, G);
+  }
   return launch_status();
 }
 
@@ -426,7 +434,7 @@ int awqmi_moe_align(const int32_t* topk_ids, int n_slots, int E, int tile_m, int
   if (n_slots <= 0 || E <= 0) return AWQMI_BAD_SHAPE;
   if (E > AWQMI_MAX_EXPERTS || tile_m <= 0 || tile_m > 4096) return AWQMI_BAD_ARGUMENT;
   const int cap = (int)awqmi_moe_align_capacity(n_slots, E, tile_m);
-  if (int st = ensure_kernel_attributes()) return st;
+  if (const int rc = ensure_kernel_attributes()) return rc;
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)(MOE_ALIGN_WAVES + 2) * E * sizeof(int),
                      (hipStream_t)stream, topk_ids, n_slots, E, tile_m, cap, sorted_token_ids,
                      expert_ids, num_tokens_post_padded);
@@ -521,7 +529,7 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
       !num_tokens_post_padded)
     return AWQMI_NULL_POINTER;
   const int G = norm_group(K, group);
-  if (int st = check_awq_shape(K, N, G)) return st;
+  if (const int rc = check_awq_shape(K, N, G)) return rc;
   if (n_slots <= 0 || E <= 0) return AWQMI_BAD_SHAPE;
   if (a_row_div <= 0 || split_k < 0 || split_k > AWQMI_MAX_SPLIT_K || E > AWQMI_MAX_EXPERTS ||
       (tile_m != 16 && tile_m != 32 && tile_m != 64 && tile_m != 128 && tile_m != 256))
@@ -538,7 +546,7 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
     if (x_rows * K * 2 >= (1ull << 32) || (size_t)K * NW * 4 >= (1ull << 32) ||
         (size_t)(K / G) * N * 2 >= (1ull << 32))
       return AWQMI_BAD_SHAPE;
-    if (int st = ensure_kernel_attributes()) return st;
+    if (const int rc = ensure_kernel_attributes()) return rc;
     MfmaGemmParams p{};
     p.x = reinterpret_cast<const half_t*>(x);
     p.qw = reinterpret_cast<const uint32_t*>(qweight);
@@ -787,7 +795,7 @@ int awqmi_fused_moe_routed_f16(const void* hidden, const float* router_logits, c
     const int valign = g_gemv_variant.load(std::memory_order_relaxed);
     if (L.n_slots >= MOE_ALIGN_SPLIT_MIN && !(valign >= 0 && (valign & 16384))) {
       // long slot lists: count per part, scan, place per part (three launches, many workgroups)
-      if (int s2 = ensure_kernel_attributes()) return s2;
+      if (const int rc = ensure_kernel_attributes()) return rc;
       int parts = (L.n_slots + 4095) / 4096;
       if (parts > MOE_ALIGN_PARTS_MAX) parts = MOE_ALIGN_PARTS_MAX;
       const int part = ((L.n_slots + parts - 1) / parts + 63) / 64 * 64;
@@ -807,17 +815,11 @@ int awqmi_fused_moe_routed_f16(const void* hidden, const float* router_logits, c
     if (st) return st;
   }
   const int Gn = norm_group(H, group);
-  if (tile == 16 && gemv_tiled_ok(H, Gn) && moe_can_fuse_act(L.n_slots, E, H, 2 * inter) &&
-      !(g_gemv_variant.load(std::memory_order_relaxed) >= 0 &&
-        (g_gemv_variant.load(std::memory_order_relaxed) & 1024))) {
-    // the w13 GEMM writes silu(gate) * up itself
-    st = moe_gemm_impl(hidden, w13_q, w13_s, w13_z, act, sorted, experts, npp, nullptr, L.n_slots, topk, 16, E, H,
-                       2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream, true);
-    if (st) return st;
-  } else if (tile == 16 && gemv_tiled_ok(H, Gn) && moe_can_fuse_act_split(L.n_slots, E, H, 2 * inter) &&
-             !(g_gemv_variant.load(std::memory_order_relaxed) >= 0 &&
-               (g_gemv_variant.load(std::memory_order_relaxed) & 1024))) {
-    // few blocks: the w13 GEMM is split in K and its last arrivers write silu(gate) * up
+  const int vact = g_gemv_variant.load(std::memory_order_relaxed);
+  if (tile == 16 && gemv_tiled_ok(H, Gn) && !(vact >= 0 && (vact & 1024)) &&
+      (moe_can_fuse_act(L.n_slots, E, H, 2 * inter) || moe_can_fuse_act_split(L.n_slots, E, H, 2 * inter))) {
+    // the w13 GEMM writes silu(gate) * up itself: in one workgroup per gate / up block pair, or,
+    // with few blocks (the launch is split in K), in the last arrivers of such a pair
     st = moe_gemm_impl(hidden, w13_q, w13_s, w13_z, act, sorted, experts, npp, nullptr, L.n_slots, topk, 16, E, H,
                        2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream, true);
     if (st) return st;

@@ -28,12 +28,12 @@ template <int ROWS>
 __global__ __launch_bounds__(256) void awq_dequant_kernel(const uint32_t* __restrict__ qw,
                                                           const half_t* __restrict__ sc,
                                                           const uint32_t* __restrict__ qz,
-                                                          half_t* __restrict__ out, int K, int NW,
-                                                          int G) {
+                                                          half_t* __restrict__ out, int k_base,
+                                                          int NW, int G) {
   const int wc = blockIdx.x * 256 + threadIdx.x;
   if (wc >= NW) return;
   const size_t N = (size_t)NW * 8;
-  const int k0 = blockIdx.y * ROWS;
+  const int k0 = k_base + blockIdx.y * ROWS;   // launches cover at most 65535 row slabs each
   const int g = k0 / G;
   const uint32_t z = qz[(size_t)g * NW + wc];
   const u4v s = *reinterpret_cast<const u4v*>(sc + (size_t)g * N + 8 * (size_t)wc);

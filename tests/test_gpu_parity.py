@@ -217,6 +217,18 @@ def test_gemm_generic_fallback(sba, gpu, M, K, N, G):
     _check_gemm(sba, gpu, x, qw, s, qz, G, 0, tag="generic")
 
 
+def test_more_rows_than_one_grid_dimension_holds(sba, gpu):
+    """Shapes whose row count exceeds 65535, the limit of a grid's second dimension: the
+    dequantize launch (one row per slab when the group size is odd) and the any-shape GEMM
+    run as consecutive slabs."""
+    _, qw, s, qz = _np_case(1, 70001, 8, 1, seed=11)
+    want = awq_ref.dequantize(qw, s, qz, 1)
+    got = sba.awq_dequantize(*_dev(gpu, qw, s, qz), 0, 0, 0).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    x, qw, s, qz = _np_case(70001, 24, 8, 8, seed=12)
+    _check_gemm(sba, gpu, x, qw, s, qz, 8, 0, tag="generic-tall")
+
+
 def test_bad_arguments_raise_without_launch(sba, gpu):
     x, qw, s, qz = _dev(gpu, *_np_case(2, 256, 64, 128, seed=1))
     with pytest.raises(ValueError):
