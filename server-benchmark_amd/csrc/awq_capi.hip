@@ -83,12 +83,12 @@ inline size_t gemv_partial_bytes(int N, int split, long long blocks_z, int tile_
   return (size_t)split * (size_t)blocks_z * tile_m * npad * sizeof(float);
 }
 
-template <int WPL, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false>
+template <int WPL, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false, bool LDSQ = false>
 void launch_gemv(const GemvParams& p, dim3 grid, hipStream_t st) {
-  if (p.G == 32) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MB, MOE, RING, KW, ACT>), grid, dim3(256), 0, st, p);
-  else if (p.G == 64) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MB, MOE, RING, KW, ACT>), grid, dim3(256), 0, st, p);
-  else if (p.G == 128) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MB, MOE, RING, KW, ACT>), grid, dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MB, MOE, RING, KW, ACT>), grid, dim3(256), 0, st, p);
+  if (p.G == 32) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 0, MB, MOE, RING, KW, ACT, LDSQ>), grid, dim3(256), 0, st, p);
+  else if (p.G == 64) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 1, MB, MOE, RING, KW, ACT, LDSQ>), grid, dim3(256), 0, st, p);
+  else if (p.G == 128) hipLaunchKernelGGL((awq_gemv_kernel<WPL, 2, MB, MOE, RING, KW, ACT, LDSQ>), grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((awq_gemv_kernel<WPL, 3, MB, MOE, RING, KW, ACT, LDSQ>), grid, dim3(256), 0, st, p);
 }
 
 // rows the skinny kernel takes in one awq_gemm call (passes of up to 32 rows)
@@ -629,7 +629,16 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   const long long runs = (long long)(nblk / p.grp) * ncg * split;
   const dim3 grid((unsigned)((runs + 7) / 8 * 8 * p.grp));
   hipStream_t st = (hipStream_t)stream;
-  if (act_pair) launch_gemv<2, 1, true, 2, 2, true>(p, grid, st);
+  // weight ring of four steps in LDS instead of two in registers, from one full block per
+  // expert on (T = 256 ... 1024 of the 128-expert block: 6 - 10 % faster; with fewer rows per
+  // expert 1 - 4 % slower, and no gain for the few-block launches once their weights come from
+  // HBM rather than from a warm cache)
+  const bool ldsq = wpl == 2 && tile_m == 16 && (size_t)K * NW * 4 < (1ull << 31) &&
+                    (long long)n_slots >= 16LL * E && !(variant >= 0 && (variant & 4096));
+  if (ldsq && act_pair) launch_gemv<2, 1, true, 4, 2, true, true>(p, grid, st);
+  else if (ldsq && pair_cols && !act_split) launch_gemv<2, 1, true, 4, 2, false, true>(p, grid, st);
+  else if (ldsq) launch_gemv<2, 1, true, 4, 4, false, true>(p, grid, st);
+  else if (act_pair) launch_gemv<2, 1, true, 2, 2, true>(p, grid, st);
   else if (act_split) launch_gemv<2, 1, true, 2>(p, grid, st);
   else if (tile_m == 32) launch_gemv<2, 2, true>(p, grid, st);
   else if (wpl == 2 && variant >= 0 && (variant & 2)) launch_gemv<2, 1, true, 4>(p, grid, st);
@@ -668,7 +677,7 @@ constexpr int MOE_ALIGN_SPLIT_MIN = 16384;   // slots from which it is used (409
 // Rows per block for the two expert GEMMs of one MoE block: 16 (the skinny kernel) or 64 /
 // 128 / 256 (the MFMA kernel's expert-grouped form).  Cost model fitted on measurements over
 // three expert shapes (2048/768 x 128 experts, 6144/2560 x 160, 4096/14336 x 8):
-//   skinny: flops / (440 TFLOP/s * avg / (avg + 24)), avg = slots per expert;
+//   skinny: flops / (540 TFLOP/s * avg / (avg + 26)), avg = slots per expert;
 //   MFMA:   per GEMM blocks * column tiles / 256 CUs rounds (a partial last round counts as
 //           at least half) of (K / 64 + overhead) k-tiles at 5.7 ns * (rows + 96) each, plus
 //           the separate SiLU pass at 4 TB/s; blocks is the expected block count after
@@ -684,7 +693,7 @@ int moe_pick_tile(int n_slots, int E, int H, int inter, int group) {
     return 16;
   const double avg = (double)n_slots / E;
   const double flops = 2.0 * n_slots * ((double)H * 2 * inter + (double)inter * H);
-  double best = flops / (440e12 * avg / (avg + 24.0));
+  double best = flops / (540e12 * avg / (avg + 26.0));
   int tile = 16;
   for (int bm : {64, 128, 256}) {
     const double blocks = avg >= bm ? (double)n_slots / bm + 0.5 * E : E * (1.0 + avg / (4.0 * bm));

@@ -98,7 +98,14 @@ struct WordVec<2> {
 //
 // MB row blocks of 16 share every B operand (MB = 2 serves up to 32 rows per pass with the
 // unpack work of one).  GMODE: 0 -> G = 32, 1 -> G = 64, 2 -> G = 128, 3 -> G = 128 * i.
-template <int WPL, int GMODE, int MB, int RING = 4>
+//
+// LDSQ: the weight ring lives in LDS instead of registers.  A 32-row step of a wave is 4 KiB
+// (32 rows x 128 bytes, WPL = 2 only); four `buffer_load_dwordx4 ... lds` instructions fetch it
+// (lane l of instruction i brings 16 bytes of row 8 i + l / 8), and the step is read back as
+// eight 8-byte LDS loads per lane right before its compute.  Ring slot d of all waves is one
+// LDS object of its own, so that the compiler's wait before reading a slot counts only the
+// loads issued after that slot's.  This buys a ring of four steps at two waves per SIMD.
+template <int WPL, int GMODE, int MB, int RING = 4, bool LDSQ = false>
 struct GemvWave {
   static constexpr int NT = 8 * WPL;                                   // 16-column tiles per wave
   static constexpr int KSPG = GMODE == 0 ? 1 : (GMODE == 1 ? 2 : 4);  // group boundaries per chunk
@@ -111,8 +118,15 @@ struct GemvWave {
   const uint32_t* qz;        // lane's zero-word pointer (wc applied)
   int NW, N, kspg, ngroups;  // kspg: 32-row steps per quantisation group
 
-  qvec q[RING][8];
+  qvec q[LDSQ ? 2 : RING][8];   // LDSQ: the step being computed and the next one, read from the LDS ring
   u4v a[RING][MB];
+  // LDSQ only
+  unsigned char* slot[RING];      // this wave's 4 KiB in each ring slot object
+  __amdgpu_buffer_rsrc_t rq;      // the (expert's) qweight as a buffer: loads past its end return 0
+  // Row r of a step sits in 128-byte line r ^ ((r >> 3) & 1) of the slot: the two 8-row
+  // blocks that one half-wave reads together then fall into different halves of the 64 banks.
+  uint32_t dma_v[2];              // lane's byte offset inside an 8-row slab, for even / odd slabs
+  uint32_t rd_off[2];             // lane's byte offset inside a slot for even / odd rows of its 8
   f4 acc[MB][NT];    // sum over finished groups of s * accg (still carrying 2^-e)
   f4 accg[MB][NT];   // current group
   qvec znext, zcur;
@@ -121,14 +135,32 @@ struct GemvWave {
   NibbleMasks nm;
 
   __device__ __forceinline__ void issue(int d, int ks) {
-    const char* rowbase = reinterpret_cast<const char*>(qw_u) + (size_t)ks * 32 * NW * 4;
+    if constexpr (LDSQ) {
+#if defined(__HIP_DEVICE_COMPILE__)
+      typedef __attribute__((address_space(3))) void lds_void;
+      const uint32_t so = (uint32_t)ks * 32u * (uint32_t)NW * 4u;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      q[d][i] = __builtin_nontemporal_load(
-          reinterpret_cast<const qvec*>(rowbase + (size_t)i * NW * 4 + q_off));
+      for (int i = 0; i < 4; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rq, (lds_void*)(slot[d] + i * 1024), 16, dma_v[i & 1],
+                                                 so + (uint32_t)i * 8u * (uint32_t)NW * 4u, 0, 0);
+#endif
+    } else {
+      const char* rowbase = reinterpret_cast<const char*>(qw_u) + (size_t)ks * 32 * NW * 4;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        q[d][i] = __builtin_nontemporal_load(
+            reinterpret_cast<const qvec*>(rowbase + (size_t)i * NW * 4 + q_off));
+    }
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
       a[d][mb] = *reinterpret_cast<const u4v*>(x_lane[mb] + (size_t)ks * 32);
+  }
+
+  // LDSQ: ring slot d -> register set d % 2
+  __device__ __forceinline__ void fetch(int d) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      q[d & 1][i] = *reinterpret_cast<const qvec*>(slot[d] + rd_off[i & 1] + (i & 6) * 128);
   }
 
   __device__ __forceinline__ int clamp_group(int step) const {
@@ -154,8 +186,8 @@ struct GemvWave {
     u4v lo, hi;
 #pragma unroll
     for (int rp = 0; rp < 4; ++rp) {
-      const uint32_t t = byte_pair<B>(WordVec<WPL>::get(q[d][2 * rp + 1], w),
-                                      WordVec<WPL>::get(q[d][2 * rp], w));
+      const uint32_t t = byte_pair<B>(WordVec<WPL>::get(q[LDSQ ? (d & 1) : d][2 * rp + 1], w),
+                                      WordVec<WPL>::get(q[LDSQ ? (d & 1) : d][2 * rp], w));
       lo[rp] = t & nm.lo;   // (w_k, w_k+1) * 2^-24 as fp16 subnormals
       hi[rp] = t & nm.hi;   // (w_k, w_k+1) * 2^-20
     }
@@ -249,6 +281,8 @@ struct GemvWave {
         adopt_group();
         if (REFILL || d + KSPG < 4) load_group(clamp_group(4 * c + d + KSPG));
       }
+      // LDSQ: the next step's weights leave the ring while this step computes
+      if (LDSQ && (REFILL || d < 3)) fetch((d + 1) % RING);
       if (GMODE == 3) {
         if (d == 0 && wide_first) {
 #pragma unroll
@@ -287,6 +321,7 @@ struct GemvWave {
     load_group(clamp_group(4 * c_begin));
 #pragma unroll
     for (int d = 0; d < RING; ++d) issue(d, 4 * c_begin + d);
+    if (LDSQ) fetch(0);
     int c = c_begin;
     for (; c + 1 < c_end; ++c) chunk<true>(c, c_begin, c_end);
     chunk<false>(c, c_begin, c_end);
@@ -305,15 +340,25 @@ struct GemvWave {
 // ACT (with KW = 2): the weight columns are [gate | up]; the workgroup takes a gate column
 // block and the up column block N / 2 columns further, and writes silu(gate) * up (both rounded
 // to fp16 first, as the unfused path stores them) to a [.., N / 2] output.
-template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false>
-__global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
+// LDSQ: weight ring of RING = 4 steps in LDS (see GemvWave), two workgroups per CU.
+template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false, bool LDSQ = false>
+__global__ __launch_bounds__(256, (RING == 4 && !LDSQ) ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
   static_assert(!ACT || (KW == 2 && MB == 1), "fused activation pairs two column blocks");
+  static_assert(!LDSQ || (WPL == 2 && RING == 4), "the LDS ring holds four steps of 128-byte rows");
   constexpr int CW = 4 / KW;       // column blocks per workgroup
   constexpr int NT = 8 * WPL;
   constexpr int CB = 128 * WPL;
-  constexpr int RS = NT * 16 + 4;  // LDS row stride in floats: 4h rows land 16 banks apart
+  // LDS row stride of the cross-wave sum in floats: padded so that 4h rows land 16 banks apart,
+  // unpadded where the two buffers take the place of ring slots 0 and 1 (16 KiB each)
+  constexpr int RS = LDSQ ? NT * 16 : NT * 16 + 4;
   constexpr int TM = 16 * MB;      // rows per pass
-  __shared__ __align__(16) float red[2][16][RS];
+  constexpr int SLOT = LDSQ ? 16384 : 16;   // bytes of one ring slot object: four waves x 4 KiB
+  __shared__ __align__(16) unsigned char lq0[SLOT], lq1[SLOT], lq2[SLOT], lq3[SLOT];
+  __shared__ __align__(16) float red_own[LDSQ ? 1 : 2][LDSQ ? 1 : 16][RS];
+  auto red = [&](int b) -> float (*)[RS] {
+    if constexpr (LDSQ) return reinterpret_cast<float (*)[RS]>(b ? lq1 : lq0);
+    else return red_own[b];
+  };
   __shared__ int s_last;
   __shared__ int s_sid[32];     // MoE: slot id of every row of this block (pads: n_slots)
   __shared__ float s_tw[32];    // MoE: routing weight of the row (1 when not applied)
@@ -361,7 +406,7 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
   int wc = cbw * (16 * WPL) + WPL * j;
   if (wc >= p.NW) wc = 0;
 
-  GemvWave<WPL, GMODE, MB, RING> w;
+  GemvWave<WPL, GMODE, MB, RING, LDSQ> w;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int r = mb * 16 + j;
@@ -375,6 +420,19 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
     w.x_lane[mb] = p.x + arow * p.K + 8 * h;
   }
   w.qw_u = qw;
+  if constexpr (LDSQ) {
+    unsigned char* const slots[4] = {lq0, lq1, lq2, lq3};
+#pragma unroll
+    for (int d = 0; d < RING; ++d) w.slot[d] = slots[d] + wave_u * 4096;
+    w.rq = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(qw), 0, (int)((size_t)p.K * p.NW * 4), 0x00020000);
+    const int wc4 = cbw * (16 * WPL) + 4 * (lane & 7);       // first of the four words this lane fetches
+    // line 8 i + l / 8 of the slot (instruction i, lane l) holds row 8 i + ((l / 8) ^ (i & 1))
+    w.dma_v[0] = (uint32_t)(((size_t)(lane >> 3) * p.NW + (wc4 < p.NW ? wc4 : 0)) * 4);
+    w.dma_v[1] = (uint32_t)(((size_t)((lane >> 3) ^ 1) * p.NW + (wc4 < p.NW ? wc4 : 0)) * 4);
+    // row 8 h + i is read from line 8 h + (i ^ (h & 1))
+    w.rd_off[0] = (uint32_t)((8 * h + (h & 1)) * 128 + 8 * j);
+    w.rd_off[1] = (uint32_t)((8 * h + (1 ^ (h & 1))) * 128 + 8 * j);
+  }
   w.q_off = (uint32_t)(((size_t)8 * h * p.NW + wc) * 4);
   w.sc = sc + 8 * (size_t)wc;
   w.qz = qz + wc;
@@ -391,6 +449,7 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
   const int c_begin = (int)(pw * nchunks / parts);
   const int c_end = (int)((pw + 1) * nchunks / parts);
   w.run(c_begin, c_end);
+  if (LDSQ) __syncthreads();   // the cross-wave sum below reuses ring slots 0 and 1
 
   const int rows_total = MOE ? s_rows : p.M;
   const size_t tile = (size_t)blk * p.ncb + cb;
@@ -412,8 +471,8 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         const int t = ww * 8 + awq_nibble_of_col(c);
-        v[c] = red[buf][m][t * 16 + jj];
-        if (two) v[c] += red[1][m][t * 16 + jj];
+        v[c] = red(buf)[m][t * 16 + jj];
+        if (two) v[c] += red(1)[m][t * 16 + jj];
       }
       size_t orow = (size_t)(mb * 16 + m);
       if (MOE) {
@@ -443,8 +502,8 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         const int t = ww * 8 + awq_nibble_of_col(c);
-        const float gv = (float)(half_t)red[0][m][t * 16 + jj];
-        const float uv = (float)(half_t)red[1][m][t * 16 + jj];
+        const float gv = (float)(half_t)red(0)[m][t * 16 + jj];
+        const float uv = (float)(half_t)red(1)[m][t * 16 + jj];
         o[c] = (half_t)(gv / (1.f + __expf(-gv)) * uv);
       }
       *reinterpret_cast<h8*>(p.y + (size_t)sid * p.ldy + col) = o;
@@ -462,7 +521,7 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
         for (int r = 0; r < 4; ++r)
           if (4 * h + r < rows) {
 #pragma unroll
-            for (int t = 0; t < NT; ++t) red[wave >> 1][4 * h + r][t * 16 + j] = w.acc[mb][t][r];
+            for (int t = 0; t < NT; ++t) red(wave >> 1)[4 * h + r][t * 16 + j] = w.acc[mb][t][r];
           }
       }
       __syncthreads();
@@ -471,7 +530,7 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
         for (int r = 0; r < 4; ++r)
           if (4 * h + r < rows) {
 #pragma unroll
-            for (int t = 0; t < NT; ++t) red[wave >> 1][4 * h + r][t * 16 + j] += w.acc[mb][t][r];
+            for (int t = 0; t < NT; ++t) red(wave >> 1)[4 * h + r][t * 16 + j] += w.acc[mb][t][r];
           }
       }
       __syncthreads();
@@ -484,14 +543,14 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
       __syncthreads();
       continue;
     }
-    // ---- cross-wave sum in LDS: red[b][row][tile*16 + j] ----
+    // ---- cross-wave sum in LDS: red(b)[row][tile*16 + j] ----
     // (rows past the block's last one are never read back)
     if (wave >= 2) {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
         if (4 * h + r < rows) {
 #pragma unroll
-          for (int t = 0; t < NT; ++t) red[wave - 2][4 * h + r][t * 16 + j] = w.acc[mb][t][r];
+          for (int t = 0; t < NT; ++t) red(wave - 2)[4 * h + r][t * 16 + j] = w.acc[mb][t][r];
         }
     }
     __syncthreads();
@@ -500,7 +559,7 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
       for (int r = 0; r < 4; ++r)
         if (4 * h + r < rows) {
 #pragma unroll
-          for (int t = 0; t < NT; ++t) red[wave][4 * h + r][t * 16 + j] += w.acc[mb][t][r];
+          for (int t = 0; t < NT; ++t) red(wave)[4 * h + r][t * 16 + j] += w.acc[mb][t][r];
         }
     }
     __syncthreads();
@@ -514,7 +573,7 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
       // neighbouring lanes write neighbouring 8-byte pairs: whole 32-byte sectors per store
       for (int i = tid * 2; i < nelem; i += 512) {
         const int m = i / (NT * 16), c = i % (NT * 16);
-        const f2 v = *reinterpret_cast<const f2*>(&red[0][m][c]) + *reinterpret_cast<const f2*>(&red[1][m][c]);
+        const f2 v = *reinterpret_cast<const f2*>(&red(0)[m][c]) + *reinterpret_cast<const f2*>(&red(1)[m][c]);
         st_coherent(mine + i, v);
       }
     } else {
@@ -570,7 +629,7 @@ __global__ __launch_bounds__(256, RING == 4 ? 1 : 2) void awq_gemv_kernel(const 
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (idx[u] < nelem) *reinterpret_cast<f2*>(&red[buf][idx[u] / (NT * 16)][idx[u] % (NT * 16)]) = v[u];
+      if (idx[u] < nelem) *reinterpret_cast<f2*>(&red(buf)[idx[u] / (NT * 16)][idx[u] % (NT * 16)]) = v[u];
   };
   if (acts) {
     const int rows = min(16, rows_total);

@@ -278,6 +278,26 @@ def test_fused_activation_agrees_with_step_by_step(sba, gpu, T):
     assert torch.equal(one, sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 8, True))
 
 
+@pytest.mark.parametrize("T,H,E,topk,I,G", [(256, 2048, 128, 8, 768, 128), (16, 1024, 16, 16, 512, 64),
+                                            (64, 512, 8, 2, 256, 32), (300, 2048, 128, 8, 768, 128),
+                                            (40, 768, 8, 4, 384, 384)])
+def test_lds_weight_ring_is_bit_identical(sba, gpu, T, H, E, topk, I, G):
+    """From one full 16-row block per expert on, the expert GEMMs keep their weight ring in LDS
+    (filled by direct-to-LDS buffer loads); with that form switched off (variant bit 4096) the
+    block must give the same bits."""
+    from server_benchmark_amd import _lib
+    lib = _lib.load()
+    assert T * topk >= 16 * E
+    c = sba.workloads.make_moe_case(T, H, E, topk, I, G, seed=T + 5).to(gpu)
+    y = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True).clone()
+    prev = lib.awqmi_set_gemv_variant(4096)
+    try:
+        y_reg = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True).clone()
+    finally:
+        lib.awqmi_set_gemv_variant(prev)
+    assert torch.equal(y.view(torch.int16), y_reg.view(torch.int16))
+
+
 @pytest.mark.parametrize("T,E,topk", [(1, 128, 8), (33, 128, 8), (7, 160, 6), (5, 16, 2)])
 def test_topk_sigmoid_with_bias(sba, gpu, T, E, topk):
     g = torch.Generator().manual_seed(T * 3 + E)

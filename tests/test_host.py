@@ -117,12 +117,11 @@ def test_fused_moe_block_rows(lib):
     """Block rows the one-call MoE entry picks: the skinny kernel's 16 for decode-sized batches,
     the MFMA kernel's 64 / 128 / 256 where measurements favoured them (points of the fit)."""
     q = lib.awqmi_fused_moe_block_rows
-    for T in (1, 16, 128, 512, 1024):
+    for T in (1, 16, 128, 512, 1024, 2048):
         assert q(T, 2048, 768, 128, 8, 128) == 16
-    assert q(2048, 2048, 768, 128, 8, 128) == 128
-    assert q(4096, 2048, 768, 128, 8, 128) == 128
+    assert q(8192, 2048, 768, 128, 8, 128) == 128
     assert q(512, 6144, 2560, 160, 8, 128) == 16
-    assert q(1024, 6144, 2560, 160, 8, 128) == 64
+    assert q(1024, 6144, 2560, 160, 8, 128) == 16
     assert q(2048, 6144, 2560, 160, 8, 128) == 128
     assert q(8192, 6144, 2560, 160, 8, 128) == 256
     assert q(64, 4096, 14336, 8, 2, 128) == 16
