@@ -22,6 +22,24 @@ namespace {
 thread_local int t_last_hip_error = 0;
 std::atomic<int> g_gemv_variant{-1};
 
+// Bits of the development switch (awqmi_set_gemv_variant; -1 = every default): each turns one
+// launch choice off, or forces one, so that two forms can be timed in one process.
+enum : int {
+  VAR_WPL1 = 1,               // one packed word per lane for every shape
+  VAR_MOE_RING4 = 2,          // MoE launches with the dense kernel's register ring of four steps
+  VAR_XCD_RUN_SHIFT = 2,      // bits 2..4 = v: force runs of 1 << (v - 1) blocks per XCD
+  VAR_NO_PAIR_COLS = 64,      // never two column blocks per workgroup
+  VAR_MFMA_FOUR_WAVES = 512,  // 64- / 128-row MFMA tiles with four waves instead of eight
+  VAR_NO_FUSED_ACT = 1024,    // the one-call MoE block always runs the separate activation kernel
+  VAR_MOE_TILE16 = 2048,      // the one-call MoE block always uses 16-row blocks
+  VAR_NO_LDS_RING = 4096,     // expert GEMMs keep the weight ring in registers
+  VAR_ALIGN_ONE_WG = 16384,   // align always in one workgroup
+};
+inline bool variant_on(int bit) {
+  const int v = g_gemv_variant.load(std::memory_order_relaxed);
+  return v >= 0 && (v & bit);
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 inline int launch_status() {
@@ -45,9 +63,7 @@ int check_awq_shape(int K, int N, int G) {
 inline bool gemv_tiled_ok(int K, int G) { return K % 128 == 0 && (G == 32 || G == 64 || G % 128 == 0); }
 
 inline int gemv_wpl(int N) {
-  const int v = g_gemv_variant.load(std::memory_order_relaxed);
-  const bool want1 = v >= 0 && (v & 1);
-  return (want1 || (N / 8) % 2 != 0) ? 1 : 2;
+  return (variant_on(VAR_WPL1) || (N / 8) % 2 != 0) ? 1 : 2;
 }
 
 // Split-K choice.  The skinny kernel runs one workgroup (one wave per SIMD, 16 KiB of loads
@@ -366,8 +382,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
       hipLaunchKernelGGL((awq_gemm_mfma_reduce_kernel<MIV, NWVV>), dim3(p.sk_tiles * MIV * (16 / NWVV)),       \
                          dim3(64 * NWVV), 0, st, p);                                              \
   } while (0)
-      const bool eight = !(g_gemv_variant.load(std::memory_order_relaxed) >= 0 &&
-                           (g_gemv_variant.load(std::memory_order_relaxed) & 512));
+      const bool eight = !variant_on(VAR_MFMA_FOUR_WAVES);
       if (mi == 1 && eight) AWQMI_MFMA(1, 8);
       else if (mi == 2 && eight) AWQMI_MFMA(2, 8);
       else if (mi == 1) AWQMI_MFMA(1, 4);
@@ -608,14 +623,14 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   // expert on, runs of 32 from 1.5 (measured on 128 experts: 6 % at one block per expert, 15 %
   // at 1.5, 3 - 4 % at 2 - 4 against runs of 8 or none; below 0.75 the order makes no difference)
   p.grp = (long long)n_slots * 2 >= 3LL * tile_m * E ? 32 : ((long long)n_slots * 4 >= 3LL * tile_m * E ? 8 : 1);
-  if (variant >= 0 && ((variant >> 2) & 7)) p.grp = 1 << (((variant >> 2) & 7) - 1);
+  if (variant >= 0 && ((variant >> VAR_XCD_RUN_SHIFT) & 7)) p.grp = 1 << (((variant >> VAR_XCD_RUN_SHIFT) & 7) - 1);
   // few chunks of K and no split across workgroups: two column blocks per workgroup, two
   // waves each (three chunks per wave at K = 768 instead of 2 / 2 / 1 / 1)
   // -- as long as the paired launch still fills the chip (blocks that will run: one per expert
   // touched or per 16 slots, whichever is more)
   const long long live_blocks = std::max<long long>((n_slots + 15) / 16, std::min(n_slots, E));
   const bool pair_cols = tile_m == 16 && wpl == 2 && split == 1 && K / 128 <= 8 && (K / 128) % 2 == 0 &&
-                         live_blocks * ((ncb + 1) / 2) >= 256 && !(variant >= 0 && (variant & 64));
+                         live_blocks * ((ncb + 1) / 2) >= 256 && !variant_on(VAR_NO_PAIR_COLS);
   // fused activation: without a split the paired-column kernel (gate and up block in one
   // workgroup); with a split the ordinary launch whose last arrivers pair the blocks up
   if (fuse_act && (wpl != 2 || tile_m != 16 || ncb % 2 != 0 || N % 512 != 0 ||
@@ -634,14 +649,14 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   // expert 1 - 4 % slower, and no gain for the few-block launches once their weights come from
   // HBM rather than from a warm cache)
   const bool ldsq = wpl == 2 && tile_m == 16 && (size_t)K * NW * 4 < (1ull << 31) &&
-                    (long long)n_slots >= 16LL * E && !(variant >= 0 && (variant & 4096));
+                    (long long)n_slots >= 16LL * E && !variant_on(VAR_NO_LDS_RING);
   if (ldsq && act_pair) launch_gemv<2, 1, true, 4, 2, true, true>(p, grid, st);
   else if (ldsq && pair_cols && !act_split) launch_gemv<2, 1, true, 4, 2, false, true>(p, grid, st);
   else if (ldsq) launch_gemv<2, 1, true, 4, 4, false, true>(p, grid, st);
   else if (act_pair) launch_gemv<2, 1, true, 2, 2, true>(p, grid, st);
   else if (act_split) launch_gemv<2, 1, true, 2>(p, grid, st);
   else if (tile_m == 32) launch_gemv<2, 2, true>(p, grid, st);
-  else if (wpl == 2 && variant >= 0 && (variant & 2)) launch_gemv<2, 1, true, 4>(p, grid, st);
+  else if (wpl == 2 && variant_on(VAR_MOE_RING4)) launch_gemv<2, 1, true, 4>(p, grid, st);
   else if (pair_cols) launch_gemv<2, 1, true, 2, 2>(p, grid, st);
   else if (wpl == 2) launch_gemv<2, 1, true, 2>(p, grid, st);
   else launch_gemv<1, 1, true>(p, grid, st);
@@ -685,8 +700,7 @@ constexpr int MOE_ALIGN_SPLIT_MIN = 16384;   // slots from which it is used (409
 // Within about 15 % of the best choice on every measured point.
 // The MFMA form also needs every operand under 4 GiB (32-bit buffer offsets).
 int moe_pick_tile(int n_slots, int E, int H, int inter, int group) {
-  const int v = g_gemv_variant.load(std::memory_order_relaxed);
-  if (v >= 0 && (v & 2048)) return 16;
+  if (variant_on(VAR_MOE_TILE16)) return 16;
   if (!gemv_tiled_ok(H, norm_group(H, group)) || !gemv_tiled_ok(inter, norm_group(inter, group))) return 16;
   if ((size_t)n_slots * std::max(H, inter) * 2 >= (1ull << 32) ||
       (size_t)H * (2 * inter / 8) * 4 >= (1ull << 32) || (size_t)inter * (H / 8) * 4 >= (1ull << 32))
@@ -801,8 +815,7 @@ int awqmi_fused_moe_routed_f16(const void* hidden, const float* router_logits, c
     st = awqmi_moe_topk_f32(router_logits, score_bias, T, E, topk, scoring, renormalize, routed_scale, ids, wts,
                             stream);
     if (st) return st;
-    const int valign = g_gemv_variant.load(std::memory_order_relaxed);
-    if (L.n_slots >= MOE_ALIGN_SPLIT_MIN && !(valign >= 0 && (valign & 16384))) {
+    if (L.n_slots >= MOE_ALIGN_SPLIT_MIN && !variant_on(VAR_ALIGN_ONE_WG)) {
       // long slot lists: count per part, scan, place per part (three launches, many workgroups)
       if (const int rc = ensure_kernel_attributes()) return rc;
       int parts = (L.n_slots + 4095) / 4096;
@@ -824,8 +837,7 @@ int awqmi_fused_moe_routed_f16(const void* hidden, const float* router_logits, c
     if (st) return st;
   }
   const int Gn = norm_group(H, group);
-  const int vact = g_gemv_variant.load(std::memory_order_relaxed);
-  if (tile == 16 && gemv_tiled_ok(H, Gn) && !(vact >= 0 && (vact & 1024)) &&
+  if (tile == 16 && gemv_tiled_ok(H, Gn) && !variant_on(VAR_NO_FUSED_ACT) &&
       (moe_can_fuse_act(L.n_slots, E, H, 2 * inter) || moe_can_fuse_act_split(L.n_slots, E, H, 2 * inter))) {
     // the w13 GEMM writes silu(gate) * up itself: in one workgroup per gate / up block pair, or,
     // with few blocks (the launch is split in K), in the last arrivers of such a pair
