@@ -34,6 +34,7 @@ enum : int {
   VAR_MOE_TILE16 = 2048,      // the one-call MoE block always uses 16-row blocks
   VAR_NO_LDS_RING = 4096,     // expert GEMMs keep the weight ring in registers
   VAR_ALIGN_ONE_WG = 16384,   // align always in one workgroup
+  VAR_MOE_TILE_SHIFT = 16,    // bits 16..17 = v: the one-call MoE block uses 64 / 128 / 256-row blocks (v = 1 / 2 / 3)
 };
 inline bool variant_on(int bit) {
   const int v = g_gemv_variant.load(std::memory_order_relaxed);
@@ -705,6 +706,8 @@ int moe_pick_tile(int n_slots, int E, int H, int inter, int group) {
   if ((size_t)n_slots * std::max(H, inter) * 2 >= (1ull << 32) ||
       (size_t)H * (2 * inter / 8) * 4 >= (1ull << 32) || (size_t)inter * (H / 8) * 4 >= (1ull << 32))
     return 16;
+  const int vv = g_gemv_variant.load(std::memory_order_relaxed);
+  if (vv >= 0 && ((vv >> VAR_MOE_TILE_SHIFT) & 3)) return 32 << ((vv >> VAR_MOE_TILE_SHIFT) & 3);
   const double avg = (double)n_slots / E;
   const double flops = 2.0 * n_slots * ((double)H * 2 * inter + (double)inter * H);
   double best = flops / (540e12 * avg / (avg + 26.0));
