@@ -136,12 +136,16 @@ def test_moe_grouped_gemm_mfma_blocks(sba, gpu, bs, T, E, topk, K, N, G):
     assert awq_ref.rel_frobenius(y2, ref2) <= TOL
 
 
-@pytest.mark.parametrize("T,H,E,topk,I", [(2048, 2048, 128, 8, 768), (1024, 1024, 8, 2, 2048),
-                                          (4096, 512, 4, 2, 384),     # many rows per expert
-                                          (640, 256, 4, 1, 1152)])    # top-1
-def test_fused_call_on_prefill_batches(sba, gpu, T, H, E, topk, I):
-    """Batches with many slots per expert, where the one-call path takes the MFMA blocks:
-    against the dense expert path and against the step-by-step path over 16-row blocks."""
+@pytest.mark.parametrize("T,H,E,topk,I,mfma", [(2048, 2048, 128, 8, 768, False), (1024, 1024, 8, 2, 2048, False),
+                                               (4096, 512, 4, 2, 384, False),     # many rows per expert
+                                               (640, 256, 4, 1, 1152, False),     # top-1
+                                               (8192, 2048, 128, 8, 768, True), (4096, 2048, 64, 6, 1408, True)])
+def test_fused_call_on_prefill_batches(sba, gpu, T, H, E, topk, I, mfma):
+    """Batches with many slots per expert, where the one-call path takes 16-row blocks with the
+    weight ring in LDS or (mfma) the MFMA kernel's 64 / 128 / 256-row blocks: against the dense
+    expert path and against the step-by-step path over 16-row blocks."""
+    from server_benchmark_amd import _lib
+    assert (_lib.load().awqmi_fused_moe_block_rows(T, H, I, E, topk, 128) >= 64) == mfma
     c = sba.workloads.make_moe_case(T, H, E, topk, I, 128, seed=T + I).to(gpu)
     one = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True)
     ref = _dense_expert_reference(sba, c, gpu, T, H, E, topk, I)
