@@ -17,6 +17,7 @@ from . import _lib
 MOE_TILE_M = 16
 _WS_COUNTER_BYTES = 65536
 _workspaces: dict = {}
+_retired: list = []      # outgrown workspaces, kept because captured graphs may still point at them
 
 
 def _stream_ptr(device) -> int:
@@ -63,6 +64,11 @@ def get_workspace(device, nbytes: int) -> torch.Tensor:
             # first GPU use in this process: the library's one-time set-up, so that no later
             # call (possibly inside a stream capture) has to do it
             _lib.check(_lib.load().awqmi_init(), "awqmi_init")
+        if ws is not None:
+            # a HIP graph captured earlier on this stream holds the old buffer's address: keep
+            # it alive, and grow geometrically so that few buffers are ever retired
+            _retired.append(ws)
+            nbytes = max(nbytes, 2 * ws.numel())
         ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
         _workspaces[key] = ws
     return ws

@@ -228,6 +228,38 @@ def test_fused_call_graph_replay(sba, gpu):
     torch.cuda.current_stream().wait_stream(s)
 
 
+def test_graph_survives_workspace_growth(sba, gpu):
+    """A graph captured with a small per-stream workspace must stay valid after a later, larger
+    call on the same stream has made the wrapper allocate a bigger one: the outgrown buffer is
+    kept alive, so the replay still finds its counters and scratch space."""
+    from server_benchmark_amd import ops
+    c = sba.workloads.make_moe_case(4, 2048, 128, 8, 768, 128, seed=9).to(gpu)
+    eager = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 8, True)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 8, True)
+        torch.cuda.synchronize()
+        small = ops.get_workspace(gpu, 1)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            y = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, 8, True)
+        big = sba.workloads.make_moe_case(3000, 2048, 128, 8, 768, 128, seed=10).to(gpu)
+        sba.fused_moe_awq(big.x, big.w13, big.w2, big.logits, 8, True)      # outgrows the workspace
+        torch.cuda.synchronize()
+        grown = ops.get_workspace(gpu, 1)
+        assert grown.data_ptr() != small.data_ptr() and grown.numel() >= 2 * small.numel()
+        del small
+        filler = torch.full((64 << 20,), 0x5A, dtype=torch.uint8, device=gpu)   # would reuse freed memory
+        for _ in range(2):
+            y.zero_()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, eager)
+        del filler
+    torch.cuda.current_stream().wait_stream(s)
+
+
 def _dense_expert_reference(sba, c, gpu, T, H, E, topk, I):
     """Every expert evaluated densely with the dequantize kernel + a library matmul."""
     w, ids = sba.topk_softmax(c.logits, topk, True)
