@@ -36,6 +36,8 @@ enum : int {
   VAR_NO_LDS_RING = 4096,     // expert GEMMs keep the weight ring in registers
   VAR_ALIGN_ONE_WG = 16384,   // align always in one workgroup
   VAR_MOE_TILE_SHIFT = 16,    // bits 16..17 = v: the one-call MoE block uses 64 / 128 / 256-row blocks (v = 1 / 2 / 3)
+  VAR_MID_M_SKINNY = 1 << 18, // awq_gemm with 17..64 rows: skinny passes wherever they can run
+  VAR_MID_M_MFMA = 1 << 19,   // awq_gemm with 17..64 rows: the MFMA kernel wherever it can run
 };
 inline bool variant_on(int bit) {
   const int v = g_gemv_variant.load(std::memory_order_relaxed);
@@ -112,12 +114,10 @@ void launch_gemv(const GemvParams& p, dim3 grid, hipStream_t st) {
 // rows the skinny kernel takes in one awq_gemm call (passes of up to 32 rows)
 constexpr int SKINNY_MAX_M = 64;
 
-// Between 33 and 64 rows two skinny passes compete with the 64-row MFMA tile: the MFMA
-// kernel wins while its tiles (times the K split) fit one round of workgroups; on very wide
-// layers, where the MFMA tiles alone fill the chip, the skinny kernel still wins up to 48 rows.
-inline bool skinny_rows(int M, int N) {
-  return M <= 32 || (M <= 48 && (N + 255) / 256 > 128);
-}
+// Up to 32 rows one skinny pass (two row blocks share every unpacked operand); from 33 rows on
+// the 64-row MFMA tile beats two skinny passes on every layer shape measured (nine shapes from
+// 2048 x 5120 to 8192 x 59136, weights read from HBM: equal at worst, up to 2 x on small layers).
+inline bool skinny_rows(int M, int /*N*/) { return M <= 32; }
 
 // Work split of the MFMA kernel: whole rounds of 256 tiles run one workgroup per tile; a
 // last round of fewer than 129 tiles (and any launch that small) is split in K over
@@ -313,8 +313,11 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   const bool mfma_ok = K % PF_BK == 0 && (((G & (G - 1)) == 0 && G >= 8) || G % 64 == 0) &&
                        mfma_slab_rows(M, K) > 0 && (size_t)K * NW * 4 < (1ull << 32) &&
                        (size_t)(K / G) * N * 2 < (1ull << 32);
+  bool mid_skinny = skinny_rows(M, N);
+  if (variant_on(VAR_MID_M_SKINNY)) mid_skinny = true;
+  if (variant_on(VAR_MID_M_MFMA)) mid_skinny = false;
   if (gemv_tiled_ok(K, G) &&
-      (M <= 16 || (M <= SKINNY_MAX_M && wpl == 2 && (skinny_rows(M, N) || !mfma_ok)))) {
+      (M <= 16 || (M <= SKINNY_MAX_M && wpl == 2 && (mid_skinny || !mfma_ok)))) {
     int split = split_k > 0 ? split_k : pick_split_k(M, K, N, G, 1);
     const int nchunks = K / 128;
     if (split > nchunks) split = nchunks;

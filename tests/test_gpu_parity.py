@@ -120,12 +120,12 @@ def test_gemm_mid_m_skinny_passes(sba, gpu, M):
     _check_gemm(sba, gpu, x, qw, s, qz, 64, 0, tag="mid-M")
 
 
-@pytest.mark.parametrize("M", [33, 48, 49, 64])
-def test_gemm_wide_layer_keeps_skinny_passes(sba, gpu, M):
-    """More than 128 column tiles: 33 .. 48 rows stay on the skinny kernel (two passes of <= 32),
-    49 .. 64 take the 64-row MFMA tile."""
+@pytest.mark.parametrize("M", [32, 33, 48, 64])
+def test_gemm_wide_layer_mid_m(sba, gpu, M):
+    """More than 128 column tiles: 32 rows run as one skinny pass, 33 .. 64 rows on the 64-row
+    MFMA tile, whose tiles alone exceed one round of workgroups here."""
     x, qw, s, qz = _np_case(M, 256, 32768 + 512, 128, seed=M)
-    _check_gemm(sba, gpu, x, qw, s, qz, 128, 0, tag="wide-skinny")
+    _check_gemm(sba, gpu, x, qw, s, qz, 128, 0, tag="wide-mid-M")
 
 
 def test_gemm_one_hot_is_exact_and_zero_weights(sba, gpu):
