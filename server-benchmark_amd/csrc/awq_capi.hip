@@ -628,6 +628,7 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   // expert on, runs of 32 from 1.5 (measured on 128 experts: 6 % at one block per expert, 15 %
   // at 1.5, 3 - 4 % at 2 - 4 against runs of 8 or none; below 0.75 the order makes no difference)
   p.grp = (long long)n_slots * 2 >= 3LL * tile_m * E ? 32 : ((long long)n_slots * 4 >= 3LL * tile_m * E ? 8 : 1);
+  if (E < 16) p.grp = 1;   // a handful of large experts: the plain order measured equal or up to 13 % faster
   if (variant >= 0 && ((variant >> VAR_XCD_RUN_SHIFT) & 7)) p.grp = 1 << (((variant >> VAR_XCD_RUN_SHIFT) & 7) - 1);
   // few chunks of K and no split across workgroups: two column blocks per workgroup, two
   // waves each (three chunks per wave at K = 768 instead of 2 / 2 / 1 / 1)
