@@ -38,6 +38,7 @@ enum : int {
   VAR_MOE_TILE_SHIFT = 16,    // bits 16..17 = v: the one-call MoE block uses 64 / 128 / 256-row blocks (v = 1 / 2 / 3)
   VAR_MID_M_SKINNY = 1 << 18, // awq_gemm with 17..64 rows: skinny passes wherever they can run
   VAR_MID_M_MFMA = 1 << 19,   // awq_gemm with 17..64 rows: the MFMA kernel wherever it can run
+  VAR_MFMA_ROWS_SHIFT = 20,   // bits 20..22 = v: MFMA tiles of 64 v rows (v = 1..4) whatever M is
 };
 inline bool variant_on(int bit) {
   const int v = g_gemv_variant.load(std::memory_order_relaxed);
@@ -131,8 +132,8 @@ inline int mfma_slab_rows(int M, int K) {
 }
 
 struct MfmaPlan { int dp_tiles, sk_tiles, sk_split; size_t part_bytes; };
-MfmaPlan plan_mfma(int M, int K, int N) {
-  const int mt = (M + PF_BM - 1) / PF_BM, nt = (N + PF_BN - 1) / PF_BN;
+MfmaPlan plan_mfma(int M, int K, int N, int bm) {
+  const int mt = (M + bm - 1) / bm, nt = (N + PF_BN - 1) / PF_BN;
   const int tiles = mt * nt, KT = K / PF_BK;
   MfmaPlan pl{tiles, 0, 1, 0};
   const int rem = tiles % 256;
@@ -146,6 +147,30 @@ MfmaPlan plan_mfma(int M, int K, int N) {
   pl.sk_split = c;
   pl.part_bytes = (size_t)rem * c * PF_SK_SLOT_FLOATS * sizeof(float);
   return pl;
+}
+
+// Rows of the MFMA tile (64, 128, 192 or 256) for one launch.  Smaller tiles pad less and give
+// more workgroups; larger ones unpack each weight for more rows.  Cost of a choice, in units of
+// one k-tile of one row: rounds of 256 workgroups (a partial last round without a K split counts
+// as at least half) x (k-tiles + 12) x (rows + 96), plus the K-split round if there is one --
+// the same per-k-tile term as in the MoE block-size choice.  Fitted on 96 points (six layer shapes,
+// M = 65 ... 2048, every tile size forced in turn): the choice is on average 0.7 % behind the best
+// size (worst point 20 %), where "256 rows from 193 rows on" was 9 % behind on average.
+int mfma_pick_rows(int M, int K, int N) {
+  if (M <= 64) return 64;
+  const int KT = K / PF_BK;
+  double best = 1e300;
+  int rows = 256;
+  for (int bm = 64; bm <= 256; bm += 64) {
+    const MfmaPlan pl = plan_mfma(M, K, N, bm);
+    const double tk = bm + 96.0;
+    const int whole = pl.dp_tiles / 256;
+    const double part = (pl.dp_tiles % 256) / 256.0;
+    double t = (whole + (part > 0 ? std::max(part, 0.5) : 0.0)) * (KT + 12) * tk;
+    if (pl.sk_tiles > 0) t += ((double)KT / pl.sk_split + 12) * tk;
+    if (t < best) { best = t; rows = bm; }
+  }
+  return rows;
 }
 
 }  // namespace
@@ -275,11 +300,9 @@ size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
   if (M > 16 && K % PF_BK == 0) {
     const int slab = mfma_slab_rows(M, K);
     if (slab > 0) {
-      mfma = plan_mfma(slab, K, N).part_bytes;
-      if (M % slab) {
-        const size_t last = plan_mfma(M % slab, K, N).part_bytes;
-        if (last > mfma) mfma = last;
-      }
+      // the tile rows the call will pick (a forced size that needs more falls back to no K split)
+      mfma = plan_mfma(slab, K, N, mfma_pick_rows(slab, K, N)).part_bytes;
+      if (M % slab) mfma = std::max(mfma, plan_mfma(M % slab, K, N, mfma_pick_rows(M % slab, K, N)).part_bytes);
     }
   }
   if (M <= SKINNY_MAX_M) {
@@ -362,11 +385,14 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
       p.M = Ms; p.K = K; p.N = N; p.NW = NW; p.G = G;
       p.gshift = 0;
       if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
-      // at most 64 / 128 / 192 rows: one row of smaller tiles instead of a padded 256-row tile
-      const int mi = Ms <= 64 ? 1 : (Ms <= 128 ? 2 : (Ms <= 192 ? 3 : 4));
-      p.mt = mi < 4 ? 1 : (Ms + PF_BM - 1) / PF_BM; p.nt = (N + PF_BN - 1) / PF_BN;
+      int mi = mfma_pick_rows(Ms, K, N) / 64;
+      const int vrows = g_gemv_variant.load(std::memory_order_relaxed);
+      if (vrows >= 0 && ((vrows >> VAR_MFMA_ROWS_SHIFT) & 7) >= 1 && ((vrows >> VAR_MFMA_ROWS_SHIFT) & 7) <= 4)
+        mi = (vrows >> VAR_MFMA_ROWS_SHIFT) & 7;
+      const int bm = 64 * mi;
+      p.mt = (Ms + bm - 1) / bm; p.nt = (N + PF_BN - 1) / PF_BN;
       p.total = p.mt * p.nt;
-      MfmaPlan pl = plan_mfma(Ms, K, N);
+      MfmaPlan pl = plan_mfma(Ms, K, N, bm);
       // the K split needs the caller's workspace (counters + partial tiles); without it every
       // tile runs on one workgroup
       if (pl.sk_tiles > 0 && (!workspace || !aligned16(workspace) ||
