@@ -201,6 +201,27 @@ def test_gemm_half_tile(sba, gpu, M, K, N, G):
     assert np.array_equal(y1.view(np.uint16), y2.view(np.uint16))
 
 
+@pytest.mark.parametrize("M,K,N,G,rows", [(257, 2048, 520, 128, None), (320, 1024, 2560, 128, None),
+                                          (384, 512, 10240, 64, None), (640, 1024, 1280, 128, None),
+                                          (700, 256, 264, 32, None),
+                                          (300, 1024, 1032, 128, 64), (300, 1024, 1032, 128, 128),
+                                          (500, 1024, 1032, 128, 192), (100, 1024, 1032, 128, 256)])
+def test_gemm_several_row_tiles_of_every_size(sba, gpu, M, K, N, G, rows):
+    """Mid-sized batches: the library picks 64-, 128-, 192- or 256-row tiles per launch and runs
+    several row tiles of the size (ragged last tile, ragged columns, K split of the last round);
+    rows forces a size through the development switch so that each one is covered."""
+    from server_benchmark_amd import _lib
+    lib = _lib.load()
+    x, qw, s, qz = _np_case(M, K, N, G, seed=M + N)
+    prev = lib.awqmi_set_gemv_variant(-1 if rows is None else (rows // 64) << 20)
+    try:
+        y1 = _check_gemm(sba, gpu, x, qw, s, qz, G, 0, tag=f"row-tiles {rows}")
+        y2 = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), 0).cpu().numpy()
+    finally:
+        lib.awqmi_set_gemv_variant(prev)
+    assert np.array_equal(y1.view(np.uint16), y2.view(np.uint16))
+
+
 @pytest.mark.parametrize("M,K,N", [(512, 1024, 1280), (300, 2048, 520), (2048, 512, 5120), (768, 1536, 8192 + 256)])
 def test_gemm_prefill_partial_rounds(sba, gpu, M, K, N):
     """Tile counts that are not a multiple of the CU count, ragged last row / column tiles;
