@@ -140,9 +140,11 @@ class SyntheticMoEDecoder:
 
     # ------------------------------------------------------------------ prefill
     @torch.no_grad()
-    def prefill(self, ids: torch.Tensor, chunk_seqs: int = 4) -> torch.Tensor:
+    def prefill(self, ids: torch.Tensor, chunk_seqs: int = 8) -> torch.Tensor:
         """ids int64 [batch, L]: fills the KV cache for positions 0..L-1 and returns the greedy
-        next token of every sequence.  Sequences are processed chunk_seqs at a time."""
+        next token of every sequence.  Sequences are processed chunk_seqs at a time (8 prompts of
+        1024 tokens = 8192 tokens per pass, the size at which the MoE block switches to the MFMA
+        kernel's 128-row blocks; measured 1.05 / 0.93 / 0.88 s for chunks of 4 / 8 / 16 prompts)."""
         cfg = self.cfg
         B, Lp = ids.shape
         assert B == self.batch and Lp < self.max_len
