@@ -152,10 +152,10 @@ MfmaPlan plan_mfma(int M, int K, int N, int bm) {
 // Rows of the MFMA tile (64, 128, 192 or 256) for one launch.  Smaller tiles pad less and give
 // more workgroups; larger ones unpack each weight for more rows.  Cost of a choice, in units of
 // one k-tile of one row: rounds of 256 workgroups (a partial last round without a K split counts
-// as at least half) x (k-tiles + 12) x (rows + 96), plus the K-split round if there is one --
-// the same per-k-tile term as in the MoE block-size choice.  Fitted on 96 points (six layer shapes,
-// M = 65 ... 2048, every tile size forced in turn): the choice is on average 0.7 % behind the best
-// size (worst point 20 %), where "256 rows from 193 rows on" was 9 % behind on average.
+// as at least 0.8) x (k-tiles + 12) x (rows + 64), plus the K-split round if there is one.
+// Fitted on 96 points (six layer shapes, M = 65 ... 2048, every tile size forced in turn, two
+// runs): the choice is within 4 % of the best size on every point (0.04 % behind on average),
+// where "256 rows from 193 rows on" was 9 % behind on average.
 int mfma_pick_rows(int M, int K, int N) {
   if (M <= 64) return 64;
   const int KT = K / PF_BK;
@@ -163,10 +163,10 @@ int mfma_pick_rows(int M, int K, int N) {
   int rows = 256;
   for (int bm = 64; bm <= 256; bm += 64) {
     const MfmaPlan pl = plan_mfma(M, K, N, bm);
-    const double tk = bm + 96.0;
+    const double tk = bm + 64.0;
     const int whole = pl.dp_tiles / 256;
     const double part = (pl.dp_tiles % 256) / 256.0;
-    double t = (whole + (part > 0 ? std::max(part, 0.5) : 0.0)) * (KT + 12) * tk;
+    double t = (whole + (part > 0 ? std::max(part, 0.8) : 0.0)) * (KT + 12) * tk;
     if (pl.sk_tiles > 0) t += ((double)KT / pl.sk_split + 12) * tk;
     if (t < best) { best = t; rows = bm; }
   }
