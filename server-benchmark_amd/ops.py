@@ -18,9 +18,18 @@ MOE_TILE_M = 16
 _WS_COUNTER_BYTES = 65536
 _workspaces: dict = {}
 _retired: list = []      # outgrown workspaces, kept because captured graphs may still point at them
+_gemm_ws_bytes: dict = {}  # (M, K, N, split) -> awqmi_gemm_workspace_bytes, asked once per shape
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream_ptr(device) -> int:
+    """Handle of torch's current stream on the device (the raw getter skips building a Stream
+    object: these wrappers run once per layer call, so a microsecond counts at M = 1)."""
+    if _raw_stream is not None:
+        idx = device.index
+        return _raw_stream(torch.cuda.current_device() if idx is None else idx)
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -52,12 +61,13 @@ def _awq_shapes(qweight, scales, qzeros, lead=0):
     return K, N, K // groups
 
 
-def get_workspace(device, nbytes: int) -> torch.Tensor:
+def get_workspace(device, nbytes: int, stream_ptr: int | None = None) -> torch.Tensor:
     """Per (device, stream) zero-initialised workspace; the kernels leave the counter
     prefix zeroed, so it is reused call after call."""
-    dev = torch.device(device)
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(),
-           torch.cuda.current_stream(dev).cuda_stream)
+    dev = device if isinstance(device, torch.device) else torch.device(device)
+    if stream_ptr is None:
+        stream_ptr = _stream_ptr(dev)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream_ptr)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         if not _workspaces:
@@ -112,11 +122,14 @@ def awq_gemm(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
         return out
     lib = _lib.load()
     split = max(0, min(int(split_k_iters), 64))
-    nbytes = lib.awqmi_gemm_workspace_bytes(M, K, N, split)
-    ws = get_workspace(input.device, nbytes)
+    shape_key = (M, K, N, split)
+    nbytes = _gemm_ws_bytes.get(shape_key)
+    if nbytes is None:
+        nbytes = _gemm_ws_bytes[shape_key] = lib.awqmi_gemm_workspace_bytes(M, K, N, split)
+    stream = _stream_ptr(input.device)
+    ws = get_workspace(input.device, nbytes, stream)
     st = lib.awqmi_gemm_f16(input.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
-                            out.data_ptr(), ws.data_ptr(), ws.numel(), M, K, N, G, split,
-                            _stream_ptr(input.device))
+                            out.data_ptr(), ws.data_ptr(), ws.numel(), M, K, N, G, split, stream)
     _lib.check(st, "awq_gemm")
     return out
 
@@ -223,11 +236,12 @@ def moe_awq_gemm(a: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, q
         out = torch.empty((n_slots, N), dtype=torch.float16, device=a.device)
     split = max(0, min(int(split_k), 64))
     nbytes = lib.awqmi_moe_gemm_workspace_bytes(n_slots, E, K, N, split, block_size)
-    ws = get_workspace(a.device, nbytes)
+    stream = _stream_ptr(a.device)
+    ws = get_workspace(a.device, nbytes, stream)
     st = lib.awqmi_moe_gemm_f16(a.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
                                 out.data_ptr(), sorted_token_ids.data_ptr(), expert_ids.data_ptr(),
                                 num_tokens_post_padded.data_ptr(), tw, n_slots, a_row_div, block_size, E, K,
-                                N, G, split, ws.data_ptr(), ws.numel(), _stream_ptr(a.device))
+                                N, G, split, ws.data_ptr(), ws.numel(), stream)
     _lib.check(st, "moe_awq_gemm")
     return out
 
@@ -298,14 +312,14 @@ def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Ten
             bias = bias_t.data_ptr()
         lib = _lib.load()
         nbytes = lib.awqmi_fused_moe_workspace_bytes(T, H, inter, E, topk)
-        ws = get_workspace(hidden_states.device, nbytes)
+        stream = _stream_ptr(hidden_states.device)
+        ws = get_workspace(hidden_states.device, nbytes, stream)
         out = torch.empty((T, H), dtype=torch.float16, device=hidden_states.device)
         st = lib.awqmi_fused_moe_routed_f16(hidden_states.data_ptr(), lg.data_ptr(), bias, w13[0].data_ptr(),
                                             w13[1].data_ptr(), w13[2].data_ptr(), w2[0].data_ptr(),
                                             w2[1].data_ptr(), w2[2].data_ptr(), out.data_ptr(), T, H, inter, E,
                                             topk, G1, 1 if scoring_func == "sigmoid" else 0, int(renormalize),
-                                            float(routed_scaling_factor), ws.data_ptr(), ws.numel(),
-                                            _stream_ptr(hidden_states.device))
+                                            float(routed_scaling_factor), ws.data_ptr(), ws.numel(), stream)
         _lib.check(st, "fused_moe_awq")
         return out
     T = hidden_states.shape[0]
