@@ -135,6 +135,9 @@ class AWQLinearMethod:
     def apply(self, layer: torch.nn.Module, x: torch.Tensor,
               bias: Optional[torch.Tensor] = None) -> torch.Tensor:
         qweight, scales, qzeros = layer.qweight, layer.scales, layer.qzeros
+        if x.dim() == 2 and x.is_contiguous():      # the decode-step case: nothing to reshape
+            out = ops.awq_gemm(x, qweight, scales, qzeros, 0)
+            return out if bias is None else out.add_(bias)
         out_shape = x.shape[:-1] + (qweight.shape[-1] * self.quant_config.pack_factor,)
         x2 = x.reshape(-1, x.shape[-1])
         if not x2.is_contiguous():
