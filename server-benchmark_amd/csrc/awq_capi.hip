@@ -33,7 +33,7 @@ enum : int {
   VAR_MFMA_FOUR_WAVES = 512,  // 64- / 128-row MFMA tiles with four waves instead of eight
   VAR_NO_FUSED_ACT = 1024,    // the one-call MoE block always runs the separate activation kernel
   VAR_MOE_TILE16 = 2048,      // the one-call MoE block always uses 16-row blocks
-  VAR_NO_LDS_RING = 4096,     // expert GEMMs keep the weight ring in registers
+  VAR_NO_LDS_RING = 4096,     // every launch keeps the weight ring in registers
   VAR_ALIGN_ONE_WG = 16384,   // align always in one workgroup
   VAR_MOE_TILE_SHIFT = 16,    // bits 16..17 = v: the one-call MoE block uses 64 / 128 / 256-row blocks (v = 1 / 2 / 3)
   VAR_MID_M_SKINNY = 1 << 18, // awq_gemm with 17..64 rows: skinny passes wherever they can run
@@ -365,7 +365,12 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
       p.x = xx + (size_t)r0 * K;
       p.y = yy + (size_t)r0 * N;
       p.M = M - r0 < 32 ? M - r0 : 32;
-      if (p.M > 16) launch_gemv<2, 2, false>(p, grid, st);
+      // 17 .. 32 rows with long wave ranges (six chunks or more): the weight ring in LDS leaves the
+      // register file to the two accumulator sets (gate_up / down_proj of the 72B shapes 3 - 11 %
+      // faster, bit-identical; short ranges measured equal or 1 - 2 % slower)
+      const bool lds32 = nchunks >= 24 * split && (size_t)K * NW * 4 < (1ull << 31) && !variant_on(VAR_NO_LDS_RING);
+      if (p.M > 16 && lds32) launch_gemv<2, 2, false, 4, 4, false, true>(p, grid, st);
+      else if (p.M > 16) launch_gemv<2, 2, false>(p, grid, st);
       else if (wpl == 2) launch_gemv<2, 1, false>(p, grid, st);
       else launch_gemv<1, 1, false>(p, grid, st);
     }

@@ -342,7 +342,7 @@ struct GemvWave {
 // to fp16 first, as the unfused path stores them) to a [.., N / 2] output.
 // LDSQ: weight ring of RING = 4 steps in LDS (see GemvWave), two workgroups per CU.
 template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false, bool LDSQ = false>
-__global__ __launch_bounds__(256, (RING == 4 && !LDSQ) ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
+__global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
   static_assert(!ACT || (KW == 2 && MB == 1), "fused activation pairs two column blocks");
   static_assert(!LDSQ || (WPL == 2 && RING == 4), "the LDS ring holds four steps of 128-byte rows");
   constexpr int CW = 4 / KW;       // column blocks per workgroup

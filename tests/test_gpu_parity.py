@@ -120,6 +120,23 @@ def test_gemm_mid_m_skinny_passes(sba, gpu, M):
     _check_gemm(sba, gpu, x, qw, s, qz, 64, 0, tag="mid-M")
 
 
+@pytest.mark.parametrize("M,K,N,G,split", [(17, 4096, 264, 128, 1), (32, 3072, 2048, 64, 1), (24, 12288, 512, 128, 0),
+                                           (32, 8192, 256, 1024, 2)])
+def test_gemm_32_row_pass_with_lds_weight_ring(sba, gpu, M, K, N, G, split):
+    """17 .. 32 rows over long wave ranges keep the weight ring in LDS; the register-ring form
+    (variant bit 4096) must give the same bits."""
+    from server_benchmark_amd import _lib
+    lib = _lib.load()
+    x, qw, s, qz = _np_case(M, K, N, G, seed=M + K)
+    y = _check_gemm(sba, gpu, x, qw, s, qz, G, split, tag="32-row lds ring")
+    prev = lib.awqmi_set_gemv_variant(4096)
+    try:
+        y_reg = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), split).cpu().numpy()
+    finally:
+        lib.awqmi_set_gemv_variant(prev)
+    assert np.array_equal(y.view(np.uint16), y_reg.view(np.uint16))
+
+
 @pytest.mark.parametrize("M", [32, 33, 48, 64])
 def test_gemm_wide_layer_mid_m(sba, gpu, M):
     """More than 128 column tiles: 32 rows run as one skinny pass, 33 .. 64 rows on the 64-row
