@@ -39,6 +39,7 @@ enum : int {
   VAR_MID_M_SKINNY = 1 << 18, // awq_gemm with 17..64 rows: skinny passes wherever they can run
   VAR_MID_M_MFMA = 1 << 19,   // awq_gemm with 17..64 rows: the MFMA kernel wherever it can run
   VAR_MFMA_ROWS_SHIFT = 20,   // bits 20..22 = v: MFMA tiles of 64 v rows (v = 1..4) whatever M is
+  VAR_NO_TAIL_STEP = 1 << 23, // dense skinny launches never share left-over chunks step by step
 };
 inline bool variant_on(int bit) {
   const int v = g_gemv_variant.load(std::memory_order_relaxed);
@@ -76,6 +77,17 @@ inline int gemv_wpl(int N) {
 // drain and refill of the memory pipeline.  So: split K just far enough that the launch is
 // one round of at most 256 workgroups, preferring a split whose 4 x split wave ranges
 // divide the 128-row chunks evenly, never below one chunk per wave.
+// Left-over chunks shared one 32-row step per wave (the kernel's TAIL form): every wave gets
+// nchunks / parts whole chunks, and the L chunks left are 4 L steps for the first 4 L waves.
+// Used for the split already chosen (down_proj of the 72B shapes, 231 chunks over 32 waves:
+// 29 steps on the busiest wave instead of 32, 1.2 - 1.9 us of 30 - 36); letting the split
+// choice count on it picked five parts for a 8192 x 10240 layer, which measured 4 % slower
+// than six without tail steps.
+inline bool gemv_tail_ok(int nchunks, int split) {
+  const int parts = 4 * split, base = nchunks / parts, left = nchunks - base * parts;
+  return base >= 1 && left > 0 && 4 * left <= parts;
+}
+
 int pick_split_k(int rows, int K, int N, int G, long long blocks_z) {
   (void)rows; (void)G;
   const int nchunks = K / 128;
@@ -102,6 +114,11 @@ inline size_t gemv_partial_bytes(int N, int split, long long blocks_z, int tile_
   if (split <= 1) return 0;
   const size_t npad = ((size_t)N + 255) / 256 * 256;
   return (size_t)split * (size_t)blocks_z * tile_m * npad * sizeof(float);
+}
+
+// dense launches of up to 16 rows with two words per lane and G = 128 can take the TAIL form
+inline bool gemv_tail_shape(int M, int N, int G) {
+  return M <= 16 && G == 128 && gemv_wpl(N) == 2 && !variant_on(VAR_NO_TAIL_STEP);
 }
 
 template <int WPL, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false, bool LDSQ = false>
@@ -371,6 +388,8 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
       const bool lds32 = nchunks >= 24 * split && (size_t)K * NW * 4 < (1ull << 31) && !variant_on(VAR_NO_LDS_RING);
       if (p.M > 16 && lds32) launch_gemv<2, 2, false, 4, 4, false, true>(p, grid, st);
       else if (p.M > 16) launch_gemv<2, 2, false>(p, grid, st);
+      else if (gemv_tail_shape(p.M, N, G) && gemv_tail_ok(nchunks, split))
+        hipLaunchKernelGGL((awq_gemv_kernel<2, 2, 1, false, 4, 4, false, false, true>), grid, dim3(256), 0, st, p);
       else if (wpl == 2) launch_gemv<2, 1, false>(p, grid, st);
       else launch_gemv<1, 1, false>(p, grid, st);
     }

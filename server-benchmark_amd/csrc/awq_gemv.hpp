@@ -105,8 +105,16 @@ struct WordVec<2> {
 // eight 8-byte LDS loads per lane right before its compute.  Ring slot d of all waves is one
 // LDS object of its own, so that the compiler's wait before reading a slot counts only the
 // loads issued after that slot's.  This buys a ring of four steps at two waves per SIMD.
-template <int WPL, int GMODE, int MB, int RING = 4, bool LDSQ = false>
+//
+// TAIL (G = 128, register ring of four): after its whole chunks the wave takes one more 32-row
+// step of a chunk that the launch's waves share step by step.  When the chunk count leaves
+// L chunks over after every wave got the same number (and 4 L <= waves), the busiest wave then
+// runs 4 n + 1 steps instead of 4 (n + 1).  The tail step goes into ring slot 0 as soon as the
+// last chunk has used it; it is a group of its own (32 rows of x against that chunk's zero
+// point and scale).  A wave without a tail step fetches a valid step and multiplies it by zeros.
+template <int WPL, int GMODE, int MB, int RING = 4, bool LDSQ = false, bool TAIL = false>
 struct GemvWave {
+  static_assert(!TAIL || (GMODE == 2 && RING == 4 && !LDSQ), "tail steps: G = 128, register ring of four");
   static constexpr int NT = 8 * WPL;                                   // 16-column tiles per wave
   static constexpr int KSPG = GMODE == 0 ? 1 : (GMODE == 1 ? 2 : 4);  // group boundaries per chunk
   typedef typename WordVec<WPL>::type qvec;
@@ -269,7 +277,7 @@ struct GemvWave {
   // No load sits behind a branch: a branch around a load makes the compiler wait for every
   // outstanding load at the join, which would empty the ring.
   template <bool REFILL>
-  __device__ __forceinline__ void chunk(int c, int c_begin, int c_end) {
+  __device__ __forceinline__ void chunk(int c, int c_begin, int c_end, int tail_step = 0) {
     bool wide_first = false;
     if (GMODE == 3) {
       const int cpg = kspg >> 2;
@@ -280,6 +288,7 @@ struct GemvWave {
       if (d % KSPG == 0) {
         adopt_group();
         if (REFILL || d + KSPG < 4) load_group(clamp_group(4 * c + d + KSPG));
+        else if (TAIL && d == 0) load_group(clamp_group(tail_step));
       }
       // LDSQ: the next step's weights leave the ring while this step computes
       if (LDSQ && (REFILL || d < 3)) fetch((d + 1) % RING);
@@ -300,6 +309,7 @@ struct GemvWave {
       // four-deep ring degenerates into load-all / wait-all / compute-all
       __builtin_amdgcn_sched_barrier(0);
       if (REFILL || d + RING < 4) issue(d % RING, 4 * c + d + RING);
+      else if (TAIL && d == 0) issue(0, tail_step);
       __builtin_amdgcn_sched_barrier(0);
       if (GMODE != 3 && (d + 1) % KSPG == 0) flush();
     }
@@ -309,7 +319,8 @@ struct GemvWave {
     }
   }
 
-  __device__ __forceinline__ void run(int c_begin, int c_end) {
+  // tail_step (TAIL only): the extra 32-row step, or -1 when this wave has none
+  __device__ __forceinline__ void run(int c_begin, int c_end, int tail_step = -1) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
@@ -324,7 +335,19 @@ struct GemvWave {
     if (LDSQ) fetch(0);
     int c = c_begin;
     for (; c + 1 < c_end; ++c) chunk<true>(c, c_begin, c_end);
-    chunk<false>(c, c_begin, c_end);
+    if constexpr (TAIL) {
+      const bool has_tail = tail_step >= 0;
+      chunk<false>(c, c_begin, c_end, has_tail ? tail_step : 4 * c);
+      adopt_group();
+      if (!has_tail) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) a[0][mb] = u4v{0u, 0u, 0u, 0u};
+      }
+      compute(0, true);
+      flush();
+    } else {
+      chunk<false>(c, c_begin, c_end);
+    }
     // undo the 2^-24 / 2^-20 carried by the low- / high-nibble tiles
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -341,10 +364,14 @@ struct GemvWave {
 // block and the up column block N / 2 columns further, and writes silu(gate) * up (both rounded
 // to fp16 first, as the unfused path stores them) to a [.., N / 2] output.
 // LDSQ: weight ring of RING = 4 steps in LDS (see GemvWave), two workgroups per CU.
-template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false, bool LDSQ = false>
+// TAIL (dense launches, see GemvWave): every wave gets the same number of whole chunks and the
+// chunks left over are taken one 32-row step per wave.
+template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false, bool LDSQ = false,
+          bool TAIL = false>
 __global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
   static_assert(!ACT || (KW == 2 && MB == 1), "fused activation pairs two column blocks");
   static_assert(!LDSQ || (WPL == 2 && RING == 4), "the LDS ring holds four steps of 128-byte rows");
+  static_assert(!TAIL || (!MOE && KW == 4 && !ACT), "tail steps are for dense launches");
   constexpr int CW = 4 / KW;       // column blocks per workgroup
   constexpr int NT = 8 * WPL;
   constexpr int CB = 128 * WPL;
@@ -406,7 +433,7 @@ __global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) voi
   int wc = cbw * (16 * WPL) + WPL * j;
   if (wc >= p.NW) wc = 0;
 
-  GemvWave<WPL, GMODE, MB, RING, LDSQ> w;
+  GemvWave<WPL, GMODE, MB, RING, LDSQ, TAIL> w;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int r = mb * 16 + j;
@@ -446,9 +473,17 @@ __global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) voi
   const long long parts = (long long)KW * p.split_k;
   const long long pw = (long long)sp * KW + wave_u % KW;
   const int nchunks = p.K / 128;
-  const int c_begin = (int)(pw * nchunks / parts);
-  const int c_end = (int)((pw + 1) * nchunks / parts);
-  w.run(c_begin, c_end);
+  if constexpr (TAIL) {
+    // the host launches this form only with at least one whole chunk per wave and at most one
+    // left-over step per wave
+    const int base = nchunks / (int)parts;
+    const int left_steps = 4 * (nchunks - base * (int)parts);
+    w.run((int)pw * base, (int)pw * base + base, pw < left_steps ? 4 * base * (int)parts + (int)pw : -1);
+  } else {
+    const int c_begin = (int)(pw * nchunks / parts);
+    const int c_end = (int)((pw + 1) * nchunks / parts);
+    w.run(c_begin, c_end);
+  }
   if (LDSQ) __syncthreads();   // the cross-wave sum below reuses ring slots 0 and 1
 
   const int rows_total = MOE ? s_rows : p.M;

@@ -109,6 +109,36 @@ def test_gemm_decode_groups_and_ragged_n(sba, gpu, K, N, G):
         _check_gemm(sba, gpu, x, qw, s, qz, g, split)
 
 
+@pytest.mark.parametrize("K,N,split,M", [(640, 256, 1, 16), (1152, 512, 1, 3), (1152, 512, 2, 16),
+                                         (4736, 256, 8, 1), (4736, 264, 8, 16), (29568, 256, 8, 7)])
+def test_gemm_decode_left_over_chunks_step_by_step(sba, gpu, K, N, split, M):
+    """Chunk counts that leave L chunks over after each of the 4 x split waves got the same
+    number, with 4 L <= waves: the left-over chunks are taken one 32-row step per wave (all
+    waves, some of them, or - N = 264 - in the one-word-per-lane form that never does).  Checked
+    against the oracle, against the whole-chunk form (variant bit 1 << 23) within tolerance, and
+    exactly with one-hot activations that sit inside the left-over chunks."""
+    from server_benchmark_amd import _lib
+    lib = _lib.load()
+    x, qw, s, qz = _np_case(M, K, N, 128, seed=K + N + split)
+    y = _check_gemm(sba, gpu, x, qw, s, qz, 128, split, tag="tail steps")
+    prev = lib.awqmi_set_gemv_variant(1 << 23)
+    try:
+        y_whole = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), split).cpu().numpy()
+    finally:
+        lib.awqmi_set_gemv_variant(prev)
+    assert awq_ref.rel_frobenius(y, y_whole.astype(np.float64)) <= 1e-3
+    W = awq_ref.dequantize(qw, s, qz, 128)
+    nchunks, parts = K // 128, 4 * split
+    first_left = (nchunks // parts) * parts * 128          # first row of the left-over chunks
+    ks = [0, first_left - 1, first_left, first_left + 31, first_left + 32, first_left + 100, K - 33, K - 1]
+    xo = np.zeros((len(ks), K), np.float16)
+    for m, k in enumerate(ks):
+        xo[m, k] = 1
+    yo = sba.awq_gemm(*_dev(gpu, xo, qw, s, qz), split).cpu().numpy()
+    for m, k in enumerate(ks):
+        assert np.array_equal(yo[m].view(np.uint16), W[k].view(np.uint16)), (m, k)
+
+
 @pytest.mark.parametrize("M", [17, 24, 32, 33, 48, 64])
 def test_gemm_mid_m_skinny_passes(sba, gpu, M):
     """17 <= M <= 64 runs the skinny kernel in passes of up to 32 rows (two row blocks share
