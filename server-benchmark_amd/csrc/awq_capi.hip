@@ -672,6 +672,7 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   p.topk_w = topk_weights; p.n_slots = n_slots; p.a_row_div = a_row_div; p.tile_m = tile_m;
   p.w_stride = (long long)K * NW; p.s_stride = (long long)(K / G) * N; p.z_stride = (long long)(K / G) * NW;
   p.nblk = nblk;
+  p.nblk_cap = (int)(awqmi_moe_align_capacity(n_slots, E, tile_m) / tile_m);
   p.ldy = fuse_act ? N / 2 : N;
   const int variant = g_gemv_variant.load(std::memory_order_relaxed);
   // group blocks by XCD once most experts have a full block: runs of 8 from 0.75 blocks per

@@ -41,6 +41,7 @@ struct GemvParams {
   int tile_m;   // rows per sorted-token block: 16 * MB
   int ldy;      // elements between output rows (N, or N / 2 when the activation is fused)
   int nblk;     // sorted-token blocks covered by the launch (a multiple of grp)
+  int nblk_cap; // blocks that sorted_ids / expert_ids hold (the align capacity; <= nblk)
   int grp;      // sorted-token blocks per XCD run
   int act_split; // split-K launch over [gate | up] columns: the last arriver of a gate block and
                  // its up block writes silu(gate) * up (one 16-row block, four waves per column block)
@@ -394,6 +395,7 @@ __global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) voi
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, h = lane >> 4;
   int cb = blockIdx.x, sp = blockIdx.y;
   int blk = 0;
+  float row_tw = 1.f;   // MoE: routing weight of row tid (threads below TM), parked in s_tw after the loop
   const uint32_t* qw = p.qw;
   const half_t* sc = p.sc;
   const uint32_t* qz = p.qz;
@@ -406,19 +408,24 @@ __global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) voi
     blk = bg * B + slot % B;
     cb = cbs / p.split_k;          // column group of the workgroup (a column block when CW = 1)
     sp = cbs % p.split_k;
-    if (blk >= p.nblk || blk * TM >= *p.n_post_pad) return;
-    const int e = p.expert_ids[blk];
+    // The block's padded count, expert and slot ids are read side by side (one trip to memory
+    // instead of three in a row; blocks past the lists' end read the last block's entries and
+    // leave right after), the routing weights behind them while the main loop runs.
+    const int blk_c = min(blk, p.nblk_cap - 1);
+    const int npp = *p.n_post_pad;
+    const int e = p.expert_ids[blk_c];
+    int sid = p.n_slots;
+    if (tid < TM) sid = p.sorted_ids[blk_c * TM + tid];
+    if (blk >= p.nblk_cap || blk * TM >= npp) return;
     qw += (size_t)e * p.w_stride;
     sc += (size_t)e * p.s_stride;
     qz += (size_t)e * p.z_stride;
     // one global read per row of the block; everything later takes ids / weights from LDS
     if (tid < 64) {
-      int sid = p.n_slots;
-      if (tid < TM) sid = p.sorted_ids[blk * TM + tid];
       const bool ok = sid < p.n_slots;
       if (tid < TM) {
         s_sid[tid] = sid;
-        s_tw[tid] = (ok && p.topk_w) ? p.topk_w[sid] : 1.f;
+        if (ok && p.topk_w) row_tw = p.topk_w[sid];
       }
       const unsigned long long m = __ballot(ok);
       if (tid == 0) s_rows = __popcll(m);   // valid slots sit at the front of a block
@@ -485,6 +492,7 @@ __global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) voi
     w.run(c_begin, c_end);
   }
   if (LDSQ) __syncthreads();   // the cross-wave sum below reuses ring slots 0 and 1
+  if (MOE && tid < TM) s_tw[tid] = row_tw;   // read behind the barriers of the cross-wave sum
 
   const int rows_total = MOE ? s_rows : p.M;
   const size_t tile = (size_t)blk * p.ncb + cb;
