@@ -389,7 +389,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
       if (p.M > 16 && lds32) launch_gemv<2, 2, false, 4, 4, false, true>(p, grid, st);
       else if (p.M > 16) launch_gemv<2, 2, false>(p, grid, st);
       else if (gemv_tail_shape(p.M, N, G) && gemv_tail_ok(nchunks, split))
-        hipLaunchKernelGGL((awq_gemv_kernel<2, 2, 1, false, 4, 4, false, false, true>), grid, dim3(256), 0, st, p);
+        hipLaunchKernelGGL((awq_gemv_tail_kernel<2, 1>), grid, dim3(256), 0, st, p);
       else if (wpl == 2) launch_gemv<2, 1, false>(p, grid, st);
       else launch_gemv<1, 1, false>(p, grid, st);
     }

@@ -367,9 +367,8 @@ struct GemvWave {
 // LDSQ: weight ring of RING = 4 steps in LDS (see GemvWave), two workgroups per CU.
 // TAIL (dense launches, see GemvWave): every wave gets the same number of whole chunks and the
 // chunks left over are taken one 32-row step per wave.
-template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false, bool LDSQ = false,
-          bool TAIL = false>
-__global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
+template <int WPL, int GMODE, int MB, bool MOE, int RING, int KW, bool ACT, bool LDSQ, bool TAIL>
+__device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
   static_assert(!ACT || (KW == 2 && MB == 1), "fused activation pairs two column blocks");
   static_assert(!LDSQ || (WPL == 2 && RING == 4), "the LDS ring holds four steps of 128-byte rows");
   static_assert(!TAIL || (!MOE && KW == 4 && !ACT), "tail steps are for dense launches");
@@ -708,6 +707,17 @@ __global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) voi
     __syncthreads();
   }
   if (tid == 0) __hip_atomic_store(p.cnt + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false, bool LDSQ = false>
+__global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
+  awq_gemv_body<WPL, GMODE, MB, MOE, RING, KW, ACT, LDSQ, false>(p);
+}
+
+// the dense G = 128 launch in its TAIL form (left-over chunks step by step)
+template <int WPL, int MB>
+__global__ __launch_bounds__(256, 1) void awq_gemv_tail_kernel(const GemvParams p) {
+  awq_gemv_body<WPL, 2, MB, false, 4, 4, false, false, true>(p);
 }
 
 }  // namespace awqmi
