@@ -173,7 +173,8 @@ struct GemvWave {
   }
 
   __device__ __forceinline__ int clamp_group(int step) const {
-    const int g = step / kspg;
+    // steps per group are a compile-time power of two except for G = 128 * i
+    const int g = GMODE == 3 ? step / kspg : step >> GMODE;
     return g < ngroups ? g : ngroups - 1;
   }
 
@@ -472,22 +473,23 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
   w.NW = p.NW;
   w.N = p.N;
   w.kspg = p.G / 32;
-  w.ngroups = p.K / p.G;
+  w.ngroups = GMODE == 3 ? p.K / p.G : p.K >> (5 + GMODE);
 
   // this wave's share of K, in 128-row chunks; the wave index is made scalar so that the
   // row base addresses stay in SGPRs
-  const long long parts = (long long)KW * p.split_k;
-  const long long pw = (long long)sp * KW + wave_u % KW;
-  const int nchunks = p.K / 128;
+  // (32-bit: at most 64 parts, K below 2^31)
+  const unsigned parts = (unsigned)KW * (unsigned)p.split_k;
+  const unsigned pw = (unsigned)sp * KW + (unsigned)wave_u % KW;
+  const int nchunks = p.K >> 7;
   if constexpr (TAIL) {
     // the host launches this form only with at least one whole chunk per wave and at most one
     // left-over step per wave
     const int base = nchunks / (int)parts;
     const int left_steps = 4 * (nchunks - base * (int)parts);
-    w.run((int)pw * base, (int)pw * base + base, pw < left_steps ? 4 * base * (int)parts + (int)pw : -1);
+    w.run((int)pw * base, (int)pw * base + base, (int)pw < left_steps ? 4 * base * (int)parts + (int)pw : -1);
   } else {
-    const int c_begin = (int)(pw * nchunks / parts);
-    const int c_end = (int)((pw + 1) * nchunks / parts);
+    const int c_begin = (int)(pw * (unsigned)nchunks / parts);
+    const int c_end = (int)((pw + 1) * (unsigned)nchunks / parts);
     w.run(c_begin, c_end);
   }
   if (LDSQ) __syncthreads();   // the cross-wave sum below reuses ring slots 0 and 1
