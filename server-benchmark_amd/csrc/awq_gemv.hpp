@@ -246,7 +246,9 @@ struct GemvWave {
       const half_t x1 = (half_t)r1;
       const half_t x2 = (half_t)(r1 - (float)x1);
       const h2 xp01 = {x0, x1}, xp2 = {x2, (half_t)0.f};
-      const h8 az = as_h8(u4v{as_u32(xp01), as_u32(xp2), 0u, 0u});
+      // (the 16-deep MFMA: its four k-slots per lane hold the three pieces and a zero, so neither
+      // operand needs zero padding registers)
+      const h4 az = __builtin_bit_cast(h4, u2v{as_u32(xp01), as_u32(xp2)});
 #pragma unroll
       for (int w = 0; w < WPL; ++w) {
         const uint32_t zw = WordVec<WPL>::get(zcur, w);
@@ -256,10 +258,10 @@ struct GemvWave {
           const uint32_t t = zbyte(zw, b);
           const uint32_t zlo = (t & nm.lo) | 0x80008000u, zhi = (t & nm.hi) | 0x80008000u;
           const int t0 = w * 8 + 2 * b;
-          accg[mb][t0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-              az, as_h8(u4v{zlo, zlo & 0x0000FFFFu, 0u, 0u}), accg[mb][t0], 0, 0, 0);
-          accg[mb][t0 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-              az, as_h8(u4v{zhi, zhi & 0x0000FFFFu, 0u, 0u}), accg[mb][t0 + 1], 0, 0, 0);
+          accg[mb][t0] = __builtin_amdgcn_mfma_f32_16x16x16f16(
+              az, __builtin_bit_cast(h4, u2v{zlo, zlo & 0x0000FFFFu}), accg[mb][t0], 0, 0, 0);
+          accg[mb][t0 + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(
+              az, __builtin_bit_cast(h4, u2v{zhi, zhi & 0x0000FFFFu}), accg[mb][t0 + 1], 0, 0, 0);
         }
       }
 #pragma unroll
