@@ -89,8 +89,12 @@ struct WordVec<2> {
 // and epilogue then overlap another workgroup's loads.
 //
 // Arithmetic.  A nibble left in place under the mask 0x000F000F (0x00F000F0) *is* the fp16
-// subnormal w * 2^-24 (w * 2^-20), and the matrix core takes subnormal fp16 inputs exactly,
-// so the B operand costs one v_perm_b32 + two v_and_b32 per four weights and no conversion.
+// subnormal w * 2^-24 (w * 2^-20), and the matrix core takes subnormal fp16 inputs exactly.
+// The high nibble w' of a byte is fed under its mask; the low nibble w is not masked at all:
+// the whole byte is the subnormal (16 w' + w) * 2^-24, its tile sums 16 x w' + x w, and the high
+// nibble's tile (the same 16 x w' * 2^-24, written as x w' * 2^-20) is subtracted when the group
+// ends - exact for one-hot rows, 16 units of fp32 rounding instead of one otherwise.  So the B
+// operand costs one v_perm_b32 + one v_and_b32 per four weights and no conversion.
 // Per quantisation group and 16-column tile the wave keeps accg = 2^-e * sum_k x_k (w_k - z):
 // the sum over w comes from the unpacked nibbles, the zero point from one more MFMA whose A
 // operand holds this lane's sum of x over the group (split into three fp16 pieces) and whose
@@ -198,8 +202,8 @@ struct GemvWave {
     for (int rp = 0; rp < 4; ++rp) {
       const uint32_t t = byte_pair<B>(WordVec<WPL>::get(q[LDSQ ? (d & 1) : d][2 * rp + 1], w),
                                       WordVec<WPL>::get(q[LDSQ ? (d & 1) : d][2 * rp], w));
-      lo[rp] = t & nm.lo;   // (w_k, w_k+1) * 2^-24 as fp16 subnormals
-      hi[rp] = t & nm.hi;   // (w_k, w_k+1) * 2^-20
+      lo[rp] = t;           // whole byte: (16 w' + w) * 2^-24 of the high- (w') and low-nibble column
+      hi[rp] = t & nm.hi;   // (w'_k, w'_k+1) * 2^-20
     }
     const int t0 = w * 8 + 2 * B;
     const f4 zero = {0.f, 0.f, 0.f, 0.f};
@@ -256,7 +260,7 @@ struct GemvWave {
         for (int b = 0; b < 4; ++b) {
           // B operand word of the zero-point MFMA: (-z, -z) * 2^-e in k-slots 0, 1 and -z in 2
           const uint32_t t = zbyte(zw, b);
-          const uint32_t zlo = (t & nm.lo) | 0x80008000u, zhi = (t & nm.hi) | 0x80008000u;
+          const uint32_t zlo = t | 0x80008000u, zhi = (t & nm.hi) | 0x80008000u;
           const int t0 = w * 8 + 2 * b;
           accg[mb][t0] = __builtin_amdgcn_mfma_f32_16x16x16f16(
               az, __builtin_bit_cast(h4, u2v{zlo, zlo & 0x0000FFFFu}), accg[mb][t0], 0, 0, 0);
@@ -271,7 +275,10 @@ struct GemvWave {
         for (int nib = 0; nib < 8; ++nib) {
           const float s = (float)sv[awq_col_of_nibble(nib)];
           const int t = w * 8 + nib;
-          acc[mb][t] += s * accg[mb][t];
+          // an even tile was fed whole bytes: its sum still holds the odd tile's column 16-fold
+          // (both in units of 2^-24, zero points included), which the odd tile's sum takes out
+          if (nib & 1) acc[mb][t] += s * accg[mb][t];
+          else acc[mb][t] += s * (accg[mb][t] - accg[mb][t + 1]);
         }
       }
     }
