@@ -34,7 +34,7 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
 # counter reads for a 256 MiB device copy; the runs are summarised in
 # profiles/awq_gemv_kernel_decode_sweep_pmc_hbm_traffic.md.  Counters cannot be read while
 # timing, so the figure is carried here and is only valid for the default split-K choice.
-DECODE_SWEEP_TRAFFIC_BYTES = 119107324
+DECODE_SWEEP_TRAFFIC_BYTES = 119090227
 
 
 def log(*a):
