@@ -58,7 +58,8 @@ def main():
     ap.add_argument("--launch", choices=("graph", "direct"), default="graph",
                     help="replay the step as a HIP graph (how a serving engine decodes) or launch directly")
     ap.add_argument("--split-k", type=int, default=0, help="0 = library heuristic")
-    ap.add_argument("--variant", type=int, default=-1, help="development: skinny-kernel variant")
+    ap.add_argument("--variant", type=int, default=-1,
+                    help="development: run the decode sweep through awqmi_dev_gemm_f16 with this launch-rule variant")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--decoder", action="store_true", help=argparse.SUPPRESS)   # kept for old command lines
@@ -88,8 +89,6 @@ def main():
         log("bench.py: no GPU visible; the HIP path has no CPU fallback")
         sys.exit(1)
     lib = _lib.load()
-    if args.variant >= 0:
-        lib.awqmi_set_gemv_variant(args.variant)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     gen = torch.Generator(device=dev).manual_seed(0)
@@ -115,9 +114,9 @@ def main():
 
     def launch(name, K, N, M, copy, stream_ptr):
         qw, sc, qz = W[name][copy]
-        st = lib.awqmi_gemm_f16(X[name][M].data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(),
-                                Y[name][M].data_ptr(), ws.data_ptr(), ws.numel(), M, K, N, G,
-                                args.split_k, stream_ptr)
+        a = (X[name][M].data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), Y[name][M].data_ptr(),
+             ws.data_ptr(), ws.numel(), M, K, N, G, args.split_k, stream_ptr)
+        st = lib.awqmi_gemm_f16(*a) if args.variant < 0 else lib.awqmi_dev_gemm_f16(*a, args.variant)
         if st != 0:
             raise RuntimeError(f"awqmi_gemm_f16 failed: {lib.awqmi_status_string(st).decode()}")
 

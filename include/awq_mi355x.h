@@ -37,7 +37,7 @@ typedef enum awqmi_status {
   AWQMI_UNSUPPORTED_GROUP = 4,   /* group size the kernels do not cover                   */
   AWQMI_LAUNCH_FAILED = 5,       /* hipGetLastError() != 0, see awqmi_last_hip_error()    */
   AWQMI_NULL_POINTER = 6,
-  AWQMI_BAD_ARGUMENT = 7         /* split_k / tile_m / topk / variant out of range        */
+  AWQMI_BAD_ARGUMENT = 7         /* split_k / tile_m / topk out of range                  */
 } awqmi_status;
 
 #define AWQMI_VERSION 100        /* major*10000 + minor*100 + patch */
@@ -180,9 +180,14 @@ int awqmi_fused_moe_routed_f16(const void* hidden_f16, const float* router_logit
                                int H, int inter, int E, int topk, int group, int scoring, int renormalize,
                                float routed_scale, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Development hook: choose among equivalent kernel variants of the skinny GEMM
- * (-1 = library default).  Returns the previous value.  Not part of the stable surface. */
-int awqmi_set_gemv_variant(int variant);
+/* Zeroes the arrival-counter prefix (AWQMI_WS_COUNTER_BYTES) of a workspace, with a small fill
+ * kernel on `stream` (no memset node: safe to capture).  Every call of this library leaves the
+ * counters at zero when its kernels run to completion; a binding calls this before it reuses a
+ * workspace after anything cut a call short: a launch that failed or was aborted (device
+ * error, a destroyed stream or graph, a process that reuses a buffer it did not zero).  No
+ * counterpart in vLLM's op surface (its split-K sums need no counters); part of the workspace
+ * contract of awqmi_gemm_f16 / awqmi_moe_gemm_f16 / awqmi_fused_moe_f16. */
+int awqmi_workspace_reset(void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

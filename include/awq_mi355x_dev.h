@@ -1,0 +1,64 @@
+/* awq_mi355x_dev.h -- development entry points of libawq_mi355x.so.
+ *
+ * Each is an entry point of awq_mi355x.h with one more argument, `variant`, that switches single
+ * launch rules of that one call off or forces them (-1 = every default, i.e. exactly the public
+ * entry point).  The variant is an argument, not a setting: it lives for the duration of the
+ * call on the calling thread and nothing else in the library can observe it, so these are as
+ * re-entrant as the calls they wrap.  They exist so that tests can push inputs through kernel
+ * forms the default rules would not pick for a small shape, and so that two forms can be timed
+ * side by side; bindings have no use for them.  They have no counterpart in the harness or in
+ * vLLM's op surface.
+ *
+ * Bits of `variant` (a value >= 0):
+ *   1        one packed word per lane in the skinny kernel for every N
+ *   2        MoE launches with the dense kernel's register ring of four steps
+ *   4|8|16   v = bits 2..4: runs of 1 << (v - 1) sorted-token blocks per XCD
+ *   64       never two column blocks per workgroup
+ *   512      64- / 128-row MFMA tiles with four waves instead of eight
+ *   1024     the one-call MoE block always runs the separate activation kernel
+ *   2048     the one-call MoE block always uses 16-row blocks
+ *   4096     every launch keeps the weight ring in registers (no LDS ring)
+ *   16384    the align step always runs in one workgroup
+ *   1 << 16  v = bits 16..17: the one-call MoE block uses 64 / 128 / 256-row blocks (v = 1 / 2 / 3)
+ *   1 << 18  awq_gemm with 17..64 rows: skinny passes wherever they can run
+ *   1 << 19  awq_gemm with 17..64 rows: the MFMA kernel wherever it can run
+ *   1 << 20  v = bits 20..22: MFMA tiles of 64 v rows (v = 1..4) whatever M is
+ *   1 << 23  dense skinny launches never share left-over chunks step by step
+ * The workspace must be large enough for the form that is forced: the sizes the public queries
+ * return cover every variant except a forced MFMA tile size, which silently runs without its K
+ * split when the workspace is too small for it.
+ */
+#ifndef AWQ_MI355X_DEV_H
+#define AWQ_MI355X_DEV_H
+
+#include "awq_mi355x.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+int awqmi_dev_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
+                       const int32_t* qzeros, void* y_f16, void* workspace, size_t workspace_bytes,
+                       int M, int K, int N, int group, int split_k, void* stream, int variant);
+
+int awqmi_dev_moe_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
+                           const int32_t* qzeros, void* y_f16, const int32_t* sorted_token_ids,
+                           const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                           const float* topk_weights, int n_slots, int a_row_div, int tile_m, int E, int K,
+                           int N, int group, int split_k, void* workspace, size_t workspace_bytes,
+                           void* stream, int variant);
+
+int awqmi_dev_fused_moe_routed_f16(const void* hidden_f16, const float* router_logits, const float* score_bias,
+                                   const int32_t* w13_qweight, const void* w13_scales_f16,
+                                   const int32_t* w13_qzeros, const int32_t* w2_qweight,
+                                   const void* w2_scales_f16, const int32_t* w2_qzeros, void* out_f16, int T,
+                                   int H, int inter, int E, int topk, int group, int scoring, int renormalize,
+                                   float routed_scale, void* workspace, size_t workspace_bytes, void* stream,
+                                   int variant);
+
+int awqmi_dev_fused_moe_block_rows(int T, int H, int inter, int E, int topk, int group, int variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AWQ_MI355X_DEV_H */

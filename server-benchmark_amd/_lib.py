@@ -10,7 +10,7 @@ LIB_PATH = os.path.join(HERE, "libawq_mi355x.so")
 
 c_int, c_void_p, c_size_t = ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 
-# name -> (restype, argtypes); mirrors include/awq_mi355x.h one to one
+# name -> (restype, argtypes); mirrors include/awq_mi355x.h and include/awq_mi355x_dev.h one to one
 SIGNATURES = {
     "awqmi_init": (c_int, []),
     "awqmi_version": (c_int, []),
@@ -40,8 +40,12 @@ SIGNATURES = {
     "awqmi_fused_moe_routed_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                            c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                            c_int, c_int, ctypes.c_float, c_void_p, c_size_t, c_void_p]),
-    "awqmi_set_gemv_variant": (c_int, [c_int]),
+    "awqmi_workspace_reset": (c_int, [c_void_p, c_size_t, c_void_p]),
 }
+# development entry points: the call they wrap plus a trailing `variant`
+for _name in ("awqmi_gemm_f16", "awqmi_moe_gemm_f16", "awqmi_fused_moe_routed_f16", "awqmi_fused_moe_block_rows"):
+    _res, _args = SIGNATURES[_name]
+    SIGNATURES[_name.replace("awqmi_", "awqmi_dev_", 1)] = (_res, [*_args, c_int])
 
 _lib = None
 

@@ -1,8 +1,8 @@
 // C ABI of libawq_mi355x.so: host-side validation and launch of the gfx950 kernels.
 // Every entry point checks its arguments before touching the device, launches on the
 // caller's stream and returns; nothing here allocates, synchronises or keeps state apart
-// from the thread-local last HIP error, the one-time kernel attribute set-up and the
-// development variant switch.  Launch shapes assume the MI355X's 256 CUs in 8 XCDs.
+// from the thread-local last HIP error and the one-time kernel attribute set-up.  Launch
+// shapes assume the MI355X's 256 CUs in 8 XCDs.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -11,6 +11,7 @@
 #include <type_traits>
 
 #include "../../include/awq_mi355x.h"
+#include "../../include/awq_mi355x_dev.h"
 #include "awq_dequant.hpp"
 #include "awq_gemm_mfma.hpp"
 #include "awq_gemv.hpp"
@@ -21,10 +22,19 @@ using namespace awqmi;
 namespace {
 
 thread_local int t_last_hip_error = 0;
-std::atomic<int> g_gemv_variant{-1};
 
-// Bits of the development switch (awqmi_set_gemv_variant; -1 = every default): each turns one
-// launch choice off, or forces one, so that two forms can be timed in one process.
+// Launch-rule variant of the call in progress on this thread: -1 (every default) for the whole
+// public C ABI; the awqmi_dev_* entry points set it for the duration of their own call only, so
+// no call can change what another call, on this thread or any other, launches.
+thread_local int t_variant = -1;
+struct VariantScope {
+  int prev;
+  explicit VariantScope(int v) : prev(t_variant) { t_variant = v; }
+  ~VariantScope() { t_variant = prev; }
+};
+
+// Bits of the `variant` argument of the awqmi_dev_* entry points: each turns one launch choice
+// off, or forces one, so that two forms can be compared and timed in one process.
 enum : int {
   VAR_WPL1 = 1,               // one packed word per lane for every shape
   VAR_MOE_RING4 = 2,          // MoE launches with the dense kernel's register ring of four steps
@@ -42,8 +52,7 @@ enum : int {
   VAR_NO_TAIL_STEP = 1 << 23, // dense skinny launches never share left-over chunks step by step
 };
 inline bool variant_on(int bit) {
-  const int v = g_gemv_variant.load(std::memory_order_relaxed);
-  return v >= 0 && (v & bit);
+  return t_variant >= 0 && (t_variant & bit);
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -272,8 +281,6 @@ const char* awqmi_status_string(int s) {
 
 int awqmi_last_hip_error(void) { return t_last_hip_error; }
 
-int awqmi_set_gemv_variant(int v) { return g_gemv_variant.exchange(v); }
-
 int awqmi_dequantize_f16(const int32_t* qweight, const void* scales, const int32_t* qzeros,
                          void* out, int K, int N, int group, void* stream) {
   if (!qweight || !scales || !qzeros || !out) return AWQMI_NULL_POINTER;
@@ -410,7 +417,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
       p.gshift = 0;
       if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
       int mi = mfma_pick_rows(Ms, K, N) / 64;
-      const int vrows = g_gemv_variant.load(std::memory_order_relaxed);
+      const int vrows = t_variant;
       if (vrows >= 0 && ((vrows >> VAR_MFMA_ROWS_SHIFT) & 7) >= 1 && ((vrows >> VAR_MFMA_ROWS_SHIFT) & 7) <= 4)
         mi = (vrows >> VAR_MFMA_ROWS_SHIFT) & 7;
       const int bm = 64 * mi;
@@ -674,7 +681,7 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   p.nblk = nblk;
   p.nblk_cap = (int)(awqmi_moe_align_capacity(n_slots, E, tile_m) / tile_m);
   p.ldy = fuse_act ? N / 2 : N;
-  const int variant = g_gemv_variant.load(std::memory_order_relaxed);
+  const int variant = t_variant;
   // group blocks by XCD once most experts have a full block: runs of 8 from 0.75 blocks per
   // expert on, runs of 32 from 1.5 (measured on 128 experts: 6 % at one block per expert, 15 %
   // at 1.5, 3 - 4 % at 2 - 4 against runs of 8 or none; below 0.75 the order makes no difference)
@@ -762,7 +769,7 @@ int moe_pick_tile(int n_slots, int E, int H, int inter, int group) {
   if ((size_t)n_slots * std::max(H, inter) * 2 >= (1ull << 32) ||
       (size_t)H * (2 * inter / 8) * 4 >= (1ull << 32) || (size_t)inter * (H / 8) * 4 >= (1ull << 32))
     return 16;
-  const int vv = g_gemv_variant.load(std::memory_order_relaxed);
+  const int vv = t_variant;
   if (vv >= 0 && ((vv >> VAR_MOE_TILE_SHIFT) & 3)) return 32 << ((vv >> VAR_MOE_TILE_SHIFT) & 3);
   const double avg = (double)n_slots / E;
   // below two 16-row blocks per expert a 64-row block is mostly padding (and the cost terms
@@ -922,6 +929,54 @@ int awqmi_fused_moe_routed_f16(const void* hidden, const float* router_logits, c
                           group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream);
   if (st) return st;
   return awqmi_moe_sum_f16(o, out, T, topk, H, stream);
+}
+
+int awqmi_workspace_reset(void* workspace, size_t workspace_bytes, void* stream) {
+  if (!workspace) return AWQMI_NULL_POINTER;
+  if (!aligned16(workspace)) return AWQMI_BAD_ALIGN;
+  if (workspace_bytes < AWQMI_WS_COUNTER_BYTES) return AWQMI_WORKSPACE_TOO_SMALL;
+  // a fill kernel rather than a memset node, so that the call behaves the same inside a capture
+  hipLaunchKernelGGL(awq_zero_words_kernel, dim3(AWQMI_WS_COUNTER_BYTES / 16 / 256), dim3(256), 0,
+                     (hipStream_t)stream, reinterpret_cast<u4v*>(workspace), AWQMI_WS_COUNTER_BYTES / 16);
+  return launch_status();
+}
+
+// ---- development entry points (include/awq_mi355x_dev.h): the same calls with the launch-rule
+// variant as an explicit argument, scoped to the call
+
+int awqmi_dev_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                       void* y, void* workspace, size_t workspace_bytes, int M, int K, int N, int group,
+                       int split_k, void* stream, int variant) {
+  VariantScope scope(variant);
+  return awqmi_gemm_f16(x, qweight, scales, qzeros, y, workspace, workspace_bytes, M, K, N, group, split_k, stream);
+}
+
+int awqmi_dev_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                           void* y, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                           const int32_t* num_tokens_post_padded, const float* topk_weights, int n_slots,
+                           int a_row_div, int tile_m, int E, int K, int N, int group, int split_k,
+                           void* workspace, size_t workspace_bytes, void* stream, int variant) {
+  VariantScope scope(variant);
+  return awqmi_moe_gemm_f16(x, qweight, scales, qzeros, y, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                            topk_weights, n_slots, a_row_div, tile_m, E, K, N, group, split_k, workspace,
+                            workspace_bytes, stream);
+}
+
+int awqmi_dev_fused_moe_routed_f16(const void* hidden, const float* router_logits, const float* score_bias,
+                                   const int32_t* w13_q, const void* w13_s, const int32_t* w13_z,
+                                   const int32_t* w2_q, const void* w2_s, const int32_t* w2_z, void* out, int T,
+                                   int H, int inter, int E, int topk, int group, int scoring, int renormalize,
+                                   float routed_scale, void* workspace, size_t workspace_bytes, void* stream,
+                                   int variant) {
+  VariantScope scope(variant);
+  return awqmi_fused_moe_routed_f16(hidden, router_logits, score_bias, w13_q, w13_s, w13_z, w2_q, w2_s, w2_z, out,
+                                    T, H, inter, E, topk, group, scoring, renormalize, routed_scale, workspace,
+                                    workspace_bytes, stream);
+}
+
+int awqmi_dev_fused_moe_block_rows(int T, int H, int inter, int E, int topk, int group, int variant) {
+  VariantScope scope(variant);
+  return awqmi_fused_moe_block_rows(T, H, inter, E, topk, group);
 }
 
 }  // extern "C"

@@ -61,4 +61,11 @@ __device__ __forceinline__ uint32_t byte_pair(uint32_t hi, uint32_t lo) {
   return __builtin_amdgcn_perm(hi, lo, sel);
 }
 
+// Fill kernel: n 16-byte words of zeros (one thread per word).  Used instead of memset nodes
+// for the arrival counters, so that a captured call replays the same way as an eager one.
+__global__ __launch_bounds__(256) void awq_zero_words_kernel(u4v* __restrict__ p, unsigned n) {
+  const unsigned i = blockIdx.x * 256u + threadIdx.x;
+  if (i < n) p[i] = u4v{0u, 0u, 0u, 0u};
+}
+
 }  // namespace awqmi

@@ -101,9 +101,16 @@ def awq_dequantize(qweight: torch.Tensor, scales: torch.Tensor, zeros: torch.Ten
 
 
 def awq_gemm(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
-             qzeros: torch.Tensor, split_k_iters: int = 0, out: torch.Tensor | None = None) -> torch.Tensor:
-    """fp16 [M, N] = input[M, K] @ dequant(qweight, scales, qzeros).  split_k_iters = 0 lets
-    the library choose; values above the library maximum are clamped."""
+             qzeros: torch.Tensor, split_k_iters: int = 0, *, force_split_k: int | None = None,
+             out: torch.Tensor | None = None, _dev_variant: int | None = None) -> torch.Tensor:
+    """fp16 [M, N] = input[M, K] @ dequant(qweight, scales, qzeros).
+
+    split_k_iters is accepted in vLLM's position and ignored, like thx / thy of awq_dequantize:
+    vLLM's AWQLinearMethod.apply always passes its pack factor (8) there, a tuning value of its
+    own kernel, and this library picks the split that fills the chip in one round of
+    workgroups from the shape.  force_split_k (1 .. 64) forces a split-K factor for the skinny
+    kernel; tests and sweeps use it.  _dev_variant routes the call through the library's
+    development entry point (single launch rules switched off or forced)."""
     _need(input, "input", torch.float16, 2)
     _need(qweight, "qweight", torch.int32, 2)
     _need(scales, "scales", torch.float16, 2)
@@ -121,17 +128,31 @@ def awq_gemm(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
     if M == 0:
         return out
     lib = _lib.load()
-    split = max(0, min(int(split_k_iters), 64))
+    split = 0 if force_split_k is None else max(0, min(int(force_split_k), 64))
     shape_key = (M, K, N, split)
     nbytes = _gemm_ws_bytes.get(shape_key)
     if nbytes is None:
         nbytes = _gemm_ws_bytes[shape_key] = lib.awqmi_gemm_workspace_bytes(M, K, N, split)
     stream = _stream_ptr(input.device)
     ws = get_workspace(input.device, nbytes, stream)
-    st = lib.awqmi_gemm_f16(input.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
-                            out.data_ptr(), ws.data_ptr(), ws.numel(), M, K, N, G, split, stream)
+    args = (input.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(), out.data_ptr(),
+            ws.data_ptr(), ws.numel(), M, K, N, G, split, stream)
+    if _dev_variant is None:
+        st = lib.awqmi_gemm_f16(*args)
+    else:
+        st = lib.awqmi_dev_gemm_f16(*args, int(_dev_variant))
     _lib.check(st, "awq_gemm")
     return out
+
+
+def reset_workspace(device=None) -> None:
+    """Zeroes the arrival counters of this (device, current stream)'s workspace.  Only needed
+    after something cut a call short (a failed or aborted launch): calls that run to completion
+    leave the counters at zero themselves."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    stream = _stream_ptr(dev)
+    ws = get_workspace(dev, 1, stream)
+    _lib.check(_lib.load().awqmi_workspace_reset(ws.data_ptr(), ws.numel(), stream), "reset_workspace")
 
 
 # --------------------------------------------------------------------------- fused MoE
@@ -202,7 +223,8 @@ def moe_awq_gemm(a: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, q
                  sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
                  num_tokens_post_padded: torch.Tensor, n_slots: int, a_row_div: int,
                  topk_weights: torch.Tensor | None = None, split_k: int = 0,
-                 out: torch.Tensor | None = None, block_size: int = MOE_TILE_M) -> torch.Tensor:
+                 out: torch.Tensor | None = None, block_size: int = MOE_TILE_M,
+                 _dev_variant: int | None = None) -> torch.Tensor:
     """Expert-grouped AWQ GEMM over blocks of `block_size` sorted slots (16 or 32: the skinny
     kernel; 64, 128 or 256: the MFMA kernel in its expert-grouped form, for many rows per expert):
     out[s] = a[s // a_row_div] @ W[expert(s)] (* topk_weights[s]).  The ids must come from
@@ -238,10 +260,13 @@ def moe_awq_gemm(a: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, q
     nbytes = lib.awqmi_moe_gemm_workspace_bytes(n_slots, E, K, N, split, block_size)
     stream = _stream_ptr(a.device)
     ws = get_workspace(a.device, nbytes, stream)
-    st = lib.awqmi_moe_gemm_f16(a.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
-                                out.data_ptr(), sorted_token_ids.data_ptr(), expert_ids.data_ptr(),
-                                num_tokens_post_padded.data_ptr(), tw, n_slots, a_row_div, block_size, E, K,
-                                N, G, split, ws.data_ptr(), ws.numel(), stream)
+    args = (a.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(), out.data_ptr(),
+            sorted_token_ids.data_ptr(), expert_ids.data_ptr(), num_tokens_post_padded.data_ptr(), tw, n_slots,
+            a_row_div, block_size, E, K, N, G, split, ws.data_ptr(), ws.numel(), stream)
+    if _dev_variant is None:
+        st = lib.awqmi_moe_gemm_f16(*args)
+    else:
+        st = lib.awqmi_dev_moe_gemm_f16(*args, int(_dev_variant))
     _lib.check(st, "moe_awq_gemm")
     return out
 
@@ -270,7 +295,7 @@ def moe_sum(x: torch.Tensor, T: int, topk: int) -> torch.Tensor:
 def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Tensor, topk: int,
                   renormalize: bool = True, block_size: int | None = None, scoring_func: str = "softmax",
                   e_score_correction_bias: torch.Tensor | None = None,
-                  routed_scaling_factor: float = 1.0) -> torch.Tensor:
+                  routed_scaling_factor: float = 1.0, _dev_variant: int | None = None) -> torch.Tensor:
     """One AWQ MoE block: route -> align -> grouped GEMM (w13) -> SiLU*up -> grouped GEMM (w2,
     scaled by the routing weight) -> sum over slots.  w13 / w2 are (qweight, scales, qzeros)
     with a leading expert dimension; w13 columns are [gate | up].  With block_size left at
@@ -315,11 +340,14 @@ def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Ten
         stream = _stream_ptr(hidden_states.device)
         ws = get_workspace(hidden_states.device, nbytes, stream)
         out = torch.empty((T, H), dtype=torch.float16, device=hidden_states.device)
-        st = lib.awqmi_fused_moe_routed_f16(hidden_states.data_ptr(), lg.data_ptr(), bias, w13[0].data_ptr(),
-                                            w13[1].data_ptr(), w13[2].data_ptr(), w2[0].data_ptr(),
-                                            w2[1].data_ptr(), w2[2].data_ptr(), out.data_ptr(), T, H, inter, E,
-                                            topk, G1, 1 if scoring_func == "sigmoid" else 0, int(renormalize),
-                                            float(routed_scaling_factor), ws.data_ptr(), ws.numel(), stream)
+        args = (hidden_states.data_ptr(), lg.data_ptr(), bias, w13[0].data_ptr(), w13[1].data_ptr(),
+                w13[2].data_ptr(), w2[0].data_ptr(), w2[1].data_ptr(), w2[2].data_ptr(), out.data_ptr(), T, H,
+                inter, E, topk, G1, 1 if scoring_func == "sigmoid" else 0, int(renormalize),
+                float(routed_scaling_factor), ws.data_ptr(), ws.numel(), stream)
+        if _dev_variant is None:
+            st = lib.awqmi_fused_moe_routed_f16(*args)
+        else:
+            st = lib.awqmi_dev_fused_moe_routed_f16(*args, int(_dev_variant))
         _lib.check(st, "fused_moe_awq")
         return out
     T = hidden_states.shape[0]
@@ -331,7 +359,9 @@ def fused_moe_awq(hidden_states: torch.Tensor, w13, w2, gating_output: torch.Ten
     # two-row-block instantiation of the skinny kernel is issue-bound)
     bs = block_size if block_size is not None else MOE_TILE_M
     sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, bs, E)
-    h13 = moe_awq_gemm(hidden_states, *w13, sorted_ids, expert_ids, npp, n, topk, block_size=bs)
+    h13 = moe_awq_gemm(hidden_states, *w13, sorted_ids, expert_ids, npp, n, topk, block_size=bs,
+                       _dev_variant=_dev_variant)
     act = silu_and_mul(h13)
-    o = moe_awq_gemm(act, *w2, sorted_ids, expert_ids, npp, n, 1, topk_weights=topk_w, block_size=bs)
+    o = moe_awq_gemm(act, *w2, sorted_ids, expert_ids, npp, n, 1, topk_weights=topk_w, block_size=bs,
+                     _dev_variant=_dev_variant)
     return moe_sum(o, T, topk)

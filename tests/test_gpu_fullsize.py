@@ -43,7 +43,7 @@ def test_decode_sizes_against_dequant_matmul(sba, gpu, name, K, N):
         print(f"[full {name}] rows of M={M} equal rows of M=16 bit for bit: {same}", flush=True)
     # split-K invariance
     for split in (1, 3, 16):
-        ys = sba.awq_gemm(x16, qw, sc, qz, split)
+        ys = sba.awq_gemm(x16, qw, sc, qz, force_split_k=split)
         assert _rel(ys, ref) <= TOL
         assert _rel(ys, y16) <= 2e-3
 

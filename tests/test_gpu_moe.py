@@ -319,18 +319,12 @@ def test_fused_activation_agrees_with_step_by_step(sba, gpu, T):
                                             (40, 768, 8, 4, 384, 384)])
 def test_lds_weight_ring_is_bit_identical(sba, gpu, T, H, E, topk, I, G):
     """From one full 16-row block per expert on, the expert GEMMs keep their weight ring in LDS
-    (filled by direct-to-LDS buffer loads); with that form switched off (variant bit 4096) the
-    block must give the same bits."""
-    from server_benchmark_amd import _lib
-    lib = _lib.load()
+    (filled by direct-to-LDS buffer loads); with that form switched off (development variant
+    bit 4096) the block must give the same bits."""
     assert T * topk >= 16 * E
     c = sba.workloads.make_moe_case(T, H, E, topk, I, G, seed=T + 5).to(gpu)
     y = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True).clone()
-    prev = lib.awqmi_set_gemv_variant(4096)
-    try:
-        y_reg = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True).clone()
-    finally:
-        lib.awqmi_set_gemv_variant(prev)
+    y_reg = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True, _dev_variant=4096).clone()
     assert torch.equal(y.view(torch.int16), y_reg.view(torch.int16))
 
 

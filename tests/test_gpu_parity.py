@@ -29,10 +29,10 @@ def _dev(dev, *arrs):
     return [torch.from_numpy(np.ascontiguousarray(a)).to(dev) for a in arrs]
 
 
-def _check_gemm(sba, dev, x, qw, s, qz, G, split_k=0, tag=""):
+def _check_gemm(sba, dev, x, qw, s, qz, G, split_k=0, tag="", variant=None):
     ref = awq_ref.gemm_wide(x, qw, s, qz, G)
     xd, qwd, sd, qzd = _dev(dev, x, qw, s, qz)
-    y = sba.awq_gemm(xd, qwd, sd, qzd, split_k)
+    y = sba.awq_gemm(xd, qwd, sd, qzd, force_split_k=split_k, _dev_variant=variant)
     torch.cuda.synchronize()
     yh = y.cpu().numpy()
     err = awq_ref.rel_frobenius(yh, ref)
@@ -89,15 +89,9 @@ def test_dequantize_exhaustive_and_fixture(sba, gpu):
 @pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("M", [1, 4, 8, 16])
 def test_gemm_decode_small(sba, gpu, M, variant):
-    from server_benchmark_amd import _lib
-    lib = _lib.load()
-    prev = lib.awqmi_set_gemv_variant(variant)
-    try:
-        x, qw, s, qz = _np_case(M, 1024, 512, 128, seed=10 + M)
-        for split in (0, 1, 2, 3, 8):
-            _check_gemm(sba, gpu, x, qw, s, qz, 128, split, tag=f"v{variant}")
-    finally:
-        lib.awqmi_set_gemv_variant(prev)
+    x, qw, s, qz = _np_case(M, 1024, 512, 128, seed=10 + M)
+    for split in (0, 1, 2, 3, 8):
+        _check_gemm(sba, gpu, x, qw, s, qz, 128, split, tag=f"v{variant}", variant=variant)
 
 
 @pytest.mark.parametrize("K,N,G", [(256, 128, 32), (256, 264, 64), (512, 136, 256), (384, 8, -1),
@@ -115,17 +109,11 @@ def test_gemm_decode_left_over_chunks_step_by_step(sba, gpu, K, N, split, M):
     """Chunk counts that leave L chunks over after each of the 4 x split waves got the same
     number, with 4 L <= waves: the left-over chunks are taken one 32-row step per wave (all
     waves, some of them, or - N = 264 - in the one-word-per-lane form that never does).  Checked
-    against the oracle, against the whole-chunk form (variant bit 1 << 23) within tolerance, and
+    against the oracle, against the whole-chunk form (development variant bit 1 << 23) within tolerance, and
     exactly with one-hot activations that sit inside the left-over chunks."""
-    from server_benchmark_amd import _lib
-    lib = _lib.load()
     x, qw, s, qz = _np_case(M, K, N, 128, seed=K + N + split)
     y = _check_gemm(sba, gpu, x, qw, s, qz, 128, split, tag="tail steps")
-    prev = lib.awqmi_set_gemv_variant(1 << 23)
-    try:
-        y_whole = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), split).cpu().numpy()
-    finally:
-        lib.awqmi_set_gemv_variant(prev)
+    y_whole = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), force_split_k=split, _dev_variant=1 << 23).cpu().numpy()
     assert awq_ref.rel_frobenius(y, y_whole.astype(np.float64)) <= 1e-3
     W = awq_ref.dequantize(qw, s, qz, 128)
     nchunks, parts = K // 128, 4 * split
@@ -134,7 +122,7 @@ def test_gemm_decode_left_over_chunks_step_by_step(sba, gpu, K, N, split, M):
     xo = np.zeros((len(ks), K), np.float16)
     for m, k in enumerate(ks):
         xo[m, k] = 1
-    yo = sba.awq_gemm(*_dev(gpu, xo, qw, s, qz), split).cpu().numpy()
+    yo = sba.awq_gemm(*_dev(gpu, xo, qw, s, qz), force_split_k=split).cpu().numpy()
     for m, k in enumerate(ks):
         assert np.array_equal(yo[m].view(np.uint16), W[k].view(np.uint16)), (m, k)
 
@@ -154,16 +142,10 @@ def test_gemm_mid_m_skinny_passes(sba, gpu, M):
                                            (32, 8192, 256, 1024, 2)])
 def test_gemm_32_row_pass_with_lds_weight_ring(sba, gpu, M, K, N, G, split):
     """17 .. 32 rows over long wave ranges keep the weight ring in LDS; the register-ring form
-    (variant bit 4096) must give the same bits."""
-    from server_benchmark_amd import _lib
-    lib = _lib.load()
+    (development variant bit 4096) must give the same bits."""
     x, qw, s, qz = _np_case(M, K, N, G, seed=M + K)
     y = _check_gemm(sba, gpu, x, qw, s, qz, G, split, tag="32-row lds ring")
-    prev = lib.awqmi_set_gemv_variant(4096)
-    try:
-        y_reg = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), split).cpu().numpy()
-    finally:
-        lib.awqmi_set_gemv_variant(prev)
+    y_reg = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), force_split_k=split, _dev_variant=4096).cpu().numpy()
     assert np.array_equal(y.view(np.uint16), y_reg.view(np.uint16))
 
 
@@ -184,7 +166,7 @@ def test_gemm_one_hot_is_exact_and_zero_weights(sba, gpu):
     for m, k in enumerate(rows):
         x[m, k] = 1
     for split in (1, 4):
-        y = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), split).cpu().numpy()
+        y = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), force_split_k=split).cpu().numpy()
         for m, k in enumerate(rows):
             assert np.array_equal(y[m].view(np.uint16), W[k].view(np.uint16)), (split, m, k)
     # w == z everywhere: the reference gives exact zeros.  The skinny kernel sums x * w on the
@@ -218,10 +200,37 @@ def test_gemm_workspace_counters_stay_zero(sba, gpu):
     x, qw, s, qz = _np_case(16, 1024, 512, 128, seed=3)
     d = _dev(gpu, x, qw, s, qz)
     for _ in range(3):
-        sba.awq_gemm(*d, 4)
+        sba.awq_gemm(*d, force_split_k=4)
     torch.cuda.synchronize()
     ws = ops.get_workspace(gpu, 1)
     assert int(ws[:65536].view(torch.int32).abs().sum().item()) == 0
+
+
+def test_workspace_reset_zeroes_the_counters(sba, gpu):
+    """A workspace whose counters were left non-zero (a call cut short) gives wrong split-K sums
+    until it is reset; awqmi_workspace_reset puts it back."""
+    from server_benchmark_amd import _lib
+    lib = _lib.load()
+    x, qw, s, qz = _np_case(16, 1024, 512, 128, seed=4)
+    xd, qwd, sd, qzd = _dev(gpu, x, qw, s, qz)
+    nbytes = lib.awqmi_gemm_workspace_bytes(16, 1024, 512, 4)
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=gpu)
+    y = torch.empty((16, 512), dtype=torch.float16, device=gpu)
+    st = torch.cuda.current_stream().cuda_stream
+
+    def call():
+        rc = lib.awqmi_gemm_f16(xd.data_ptr(), qwd.data_ptr(), sd.data_ptr(), qzd.data_ptr(), y.data_ptr(),
+                                ws.data_ptr(), ws.numel(), 16, 1024, 512, 128, 4, st)
+        assert rc == 0
+        torch.cuda.synchronize()
+        return y.clone()
+
+    good = call()
+    ws[:65536].view(torch.int32).fill_(-7)      # what a launch that died half-way could leave behind
+    assert lib.awqmi_workspace_reset(ws.data_ptr(), ws.numel(), st) == 0
+    torch.cuda.synchronize()
+    assert int(ws[:65536].view(torch.int32).abs().sum().item()) == 0
+    assert torch.equal(call(), good)
 
 
 # ------------------------------------------------------------------ prefill GEMM (M > 16) and fallback
@@ -256,16 +265,11 @@ def test_gemm_half_tile(sba, gpu, M, K, N, G):
 def test_gemm_several_row_tiles_of_every_size(sba, gpu, M, K, N, G, rows):
     """Mid-sized batches: the library picks 64-, 128-, 192- or 256-row tiles per launch and runs
     several row tiles of the size (ragged last tile, ragged columns, K split of the last round);
-    rows forces a size through the development switch so that each one is covered."""
-    from server_benchmark_amd import _lib
-    lib = _lib.load()
+    rows forces a size through the development entry point so that each one is covered."""
     x, qw, s, qz = _np_case(M, K, N, G, seed=M + N)
-    prev = lib.awqmi_set_gemv_variant(-1 if rows is None else (rows // 64) << 20)
-    try:
-        y1 = _check_gemm(sba, gpu, x, qw, s, qz, G, 0, tag=f"row-tiles {rows}")
-        y2 = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), 0).cpu().numpy()
-    finally:
-        lib.awqmi_set_gemv_variant(prev)
+    variant = None if rows is None else (rows // 64) << 20
+    y1 = _check_gemm(sba, gpu, x, qw, s, qz, G, 0, tag=f"row-tiles {rows}", variant=variant)
+    y2 = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), 0, _dev_variant=variant).cpu().numpy()
     assert np.array_equal(y1.view(np.uint16), y2.view(np.uint16))
 
 

@@ -21,7 +21,10 @@ def lib():
 
 def test_library_exports_every_declared_symbol(lib):
     from server_benchmark_amd import _lib
-    hdr = open(os.path.join(ROOT, "include", "awq_mi355x.h")).read()
+    hdr = ""
+    for name in sorted(os.listdir(os.path.join(ROOT, "include"))):
+        if name.endswith(".h"):
+            hdr += open(os.path.join(ROOT, "include", name)).read()
     hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
     declared = set(re.findall(r"\b(awqmi_[a-z0-9_]+)\s*\(", hdr))
     assert len(declared) >= 14
@@ -84,6 +87,24 @@ def test_validation_happens_before_any_launch(lib):
     assert lib.awqmi_fused_moe_routed_f16(*okr, 4, 256, 128, 8, 2, 128, 2, 1, 1.0, fake, 1 << 30, 0) == 7
     assert lib.awqmi_fused_moe_routed_f16(*okr, 4, 256, 128, 8, 2, 128, 1, 1, 2.5, fake, 1024, 0) == 3
     assert lib.awqmi_fused_moe_f16(*ok, 4, 250, 128, 8, 2, 128, 1, fake, 1 << 30, 0) == 1
+
+
+def test_workspace_reset_and_dev_entry_points_validate_on_the_host(lib):
+    fake, odd = 0x1000, 0x1008
+    assert lib.awqmi_workspace_reset(0, 1 << 20, 0) == 6
+    assert lib.awqmi_workspace_reset(odd, 1 << 20, 0) == 2
+    assert lib.awqmi_workspace_reset(fake, 65535, 0) == 3
+    # the development entry points are the public ones plus a variant argument: same checks,
+    # and the variant of one call is gone when the call returns (the query that follows sees
+    # the default rules again)
+    assert lib.awqmi_dev_gemm_f16(fake, fake, fake, fake, 0, 0, 0, 1, 128, 64, 128, 0, 0, 1) == 6
+    assert lib.awqmi_dev_gemm_f16(fake, fake, fake, fake, fake, 0, 0, 4, 1024, 64, 128, 65, 0, 1 << 23) == 7
+    big = (4096, 2048, 768, 128, 8, 128)
+    rows = lib.awqmi_fused_moe_block_rows(*big)
+    assert lib.awqmi_dev_fused_moe_block_rows(*big, 2048) == 16
+    assert lib.awqmi_dev_fused_moe_block_rows(*big, 2 << 16) == 128
+    assert lib.awqmi_dev_fused_moe_block_rows(*big, -1) == rows
+    assert lib.awqmi_fused_moe_block_rows(*big) == rows
 
 
 def test_fused_moe_workspace_covers_every_intermediate(lib):
