@@ -37,7 +37,8 @@ typedef enum awqmi_status {
   AWQMI_UNSUPPORTED_GROUP = 4,   /* group size the kernels do not cover                   */
   AWQMI_LAUNCH_FAILED = 5,       /* hipGetLastError() != 0, see awqmi_last_hip_error()    */
   AWQMI_NULL_POINTER = 6,
-  AWQMI_BAD_ARGUMENT = 7         /* split_k / tile_m / topk out of range                  */
+  AWQMI_BAD_ARGUMENT = 7,        /* split_k / tile_m / topk out of range                  */
+  AWQMI_SCRATCH_LIMIT = 8        /* awqmi_gemm_f16_noalloc: needs > AWQMI_STATIC_SCRATCH_BYTES */
 } awqmi_status;
 
 #define AWQMI_VERSION 100        /* major*10000 + minor*100 + patch */
@@ -46,8 +47,10 @@ typedef enum awqmi_status {
 #define AWQMI_MAX_EXPERTS 1024
 
 /* Optional one-time set-up on the current device: raises the dynamic-LDS limit of the kernels
- * that need it.  Every entry point does the same on its first use; call this once after
- * loading the library if the first use may sit inside a stream capture.  The library assumes
+ * that need it, looks up this GPU's static scratch array (awqmi_gemm_f16_noalloc) and zeroes its
+ * arrival counters (synchronously, on the null stream).  Every entry point does its share of
+ * this on its first use; call this once after loading the library if the first use may sit
+ * inside a stream capture.  The library assumes
  * one GPU per process (the harness starts one server process per replica and GPU set,
  * reference utils/generate_compose.py:85-100). */
 int awqmi_init(void);
@@ -89,6 +92,32 @@ size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k);
 int awqmi_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
                    const int32_t* qzeros, void* y_f16, void* workspace, size_t workspace_bytes,
                    int M, int K, int N, int group, int split_k, void* stream);
+
+/* awqmi_gemm_f16 for callers that cannot allocate or carry a workspace: code under HIP graph
+ * capture that has no buffer of its own, tight serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the harness or in vLLM's op surface (vLLM's awq_gemm allocates its
+ * split-K buffer per call through torch).  Same arguments as awqmi_gemm_f16 minus the
+ * workspace; the split-K arrival counters and fp32 partial tiles live in a static device array
+ * of AWQMI_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process
+ * ends), and results are bit-identical to awqmi_gemm_f16 with a zeroed workspace of that many
+ * bytes.  The call allocates and frees nothing.
+ *   - Rows up to 32 (the skinny kernel): a call whose split-K partial tiles do not fit returns
+ *     AWQMI_SCRATCH_LIMIT and launches nothing.  With split_k = 0 every shape fits (at most
+ *     8 MiB + the counters); only a large forced split_k on a wide layer does not.
+ *   - More rows (the MFMA kernel): when the partial tiles of its K split do not fit, every
+ *     tile runs on one workgroup, as awqmi_gemm_f16 does with a workspace of that size.
+ *   - All calls on one GPU share that GPU's array: two calls that overlap in time on one GPU
+ *     (different streams, or graphs replayed side by side) race on it; serialise them or give
+ *     the others awqmi_gemm_f16 with their own workspace.
+ *   - The array keeps the last call's partial tiles; only the counters must start at zero.
+ *     They are zero when the library is loaded and every call that runs to completion leaves
+ *     them so; awqmi_init() zeroes them again (use it after a call that was cut short).
+ *   - The device address of the array is looked up on the first call on each GPU (or by
+ *     awqmi_init() with that GPU current); the stream must belong to the current device. */
+#define AWQMI_STATIC_SCRATCH_BYTES (AWQMI_WS_COUNTER_BYTES + (16u << 20))
+int awqmi_gemm_f16_noalloc(const void* x_f16, const int32_t* qweight, const void* scales_f16,
+                           const int32_t* qzeros, void* y_f16, int M, int K, int N, int group,
+                           int split_k, void* stream);
 
 /* Router: softmax over E experts, top-k (ties: lowest expert id), optional renormalise.
  * Stands in for the fused-MoE routing step of the MoE AWQ models at reference

@@ -21,6 +21,8 @@ SIGNATURES = {
     "awqmi_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "awqmi_gemm_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "awqmi_gemm_f16_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                       c_int, c_void_p]),
     "awqmi_moe_topk_softmax_f32": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "awqmi_moe_topk_f32": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, ctypes.c_float, c_void_p,
                                    c_void_p, c_void_p]),
@@ -81,6 +83,6 @@ def check(status: int, what: str):
     msg = lib.awqmi_status_string(status).decode()
     if status == 5:
         raise AWQKernelError(f"{what}: {msg} (hipError {lib.awqmi_last_hip_error()})")
-    if status in (1, 2, 4, 6, 7):
+    if status in (1, 2, 4, 6, 7, 8):
         raise ValueError(f"{what}: {msg}")
     raise AWQKernelError(f"{what}: {msg}")

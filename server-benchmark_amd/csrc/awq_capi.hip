@@ -19,6 +19,13 @@
 
 using namespace awqmi;
 
+// Scratch of the allocation-free entry point (awqmi_gemm_f16_noalloc): split-K arrival counters
+// (the first AWQMI_WS_COUNTER_BYTES) and fp32 partial tiles.  Every GPU the library runs on
+// holds its own copy of this array at its own address until the process ends.  The name below
+// is a host-side stand-in, not a device address: host code only ever uses the pointer that
+// hipGetSymbolAddress returned for the current device (static_scratch_ptr).
+static __device__ __align__(256) unsigned char scratch[AWQMI_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local int t_last_hip_error = 0;
@@ -56,6 +63,25 @@ inline bool variant_on(int bit) {
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Device address of `scratch` on the current GPU, looked up once per device.
+constexpr int MAX_DEVICES = 64;
+std::atomic<void*> g_scratch_ptr[MAX_DEVICES];
+int static_scratch_ptr(void** out, bool* first_use) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
+  if (dev < 0 || dev >= MAX_DEVICES) return AWQMI_BAD_ARGUMENT;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  *first_use = ptr == nullptr;
+  if (!ptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return AWQMI_OK;
+}
 
 inline int launch_status() {
   const hipError_t e = hipGetLastError();
@@ -261,7 +287,21 @@ static int moe_route_align_small(const float* logits, int T, int E, int topk, in
 
 extern "C" {
 
-int awqmi_init(void) { return ensure_kernel_attributes(); }
+int awqmi_init(void) {
+  if (const int rc = ensure_kernel_attributes()) return rc;
+  // the current device's static scratch array: look its address up and put its arrival counters
+  // at zero (they are zero when the code object is loaded and every completed call leaves them
+  // so; calling this again is the way back after a call that was cut short)
+  void* ptr = nullptr;
+  bool first = false;
+  if (const int rc = static_scratch_ptr(&ptr, &first)) return rc;
+  hipLaunchKernelGGL(awq_zero_words_kernel, dim3(AWQMI_WS_COUNTER_BYTES / 16 / 256), dim3(256), 0, (hipStream_t) nullptr,
+                     reinterpret_cast<u4v*>(ptr), AWQMI_WS_COUNTER_BYTES / 16);
+  if (const int rc = launch_status()) return rc;
+  const hipError_t e = hipStreamSynchronize(nullptr);
+  if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
+  return AWQMI_OK;
+}
 
 int awqmi_version(void) { return AWQMI_VERSION; }
 
@@ -275,6 +315,9 @@ const char* awqmi_status_string(int s) {
     case AWQMI_LAUNCH_FAILED: return "kernel launch failed";
     case AWQMI_NULL_POINTER: return "null pointer";
     case AWQMI_BAD_ARGUMENT: return "bad argument";
+    case AWQMI_SCRATCH_LIMIT:
+      return "call needs more scratch than the static array holds (AWQMI_STATIC_SCRATCH_BYTES); "
+             "use awqmi_gemm_f16 with a caller-owned workspace";
     default: return "unknown status";
   }
 }
@@ -464,6 +507,18 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
                        xx + (size_t)r0 * K, qw, sc, qz, yy + (size_t)r0 * N, Ms, K, NW, G);
   }
   return launch_status();
+}
+
+int awqmi_gemm_f16_noalloc(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                           void* y, int M, int K, int N, int group, int split_k, void* stream) {
+  void* ptr = nullptr;
+  bool first = false;
+  if (const int rc = static_scratch_ptr(&ptr, &first)) return rc;
+  // exactly awqmi_gemm_f16 with this GPU's static array as the workspace (it validates before
+  // it launches, so a skinny call whose split-K partial tiles do not fit launches nothing)
+  const int rc = awqmi_gemm_f16(x, qweight, scales, qzeros, y, ptr, AWQMI_STATIC_SCRATCH_BYTES, M, K, N, group,
+                                split_k, stream);
+  return rc == AWQMI_WORKSPACE_TOO_SMALL ? AWQMI_SCRATCH_LIMIT : rc;
 }
 
 int awqmi_moe_topk_f32(const float* logits, const float* score_bias, int T, int E, int topk, int scoring,

@@ -145,6 +145,31 @@ def awq_gemm(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
     return out
 
 
+def awq_gemm_noalloc(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, qzeros: torch.Tensor,
+                     out: torch.Tensor, force_split_k: int | None = None) -> torch.Tensor:
+    """awq_gemm into a caller-provided `out` through the library's allocation-free entry point:
+    split-K counters and partial tiles live in a static device array inside the library, so
+    neither this wrapper nor the library allocates.  All such calls on one GPU share that array
+    and must not overlap in time.  Raises ValueError when the call's split-K tiles do not fit."""
+    _need(input, "input", torch.float16, 2)
+    _need(qweight, "qweight", torch.int32, 2)
+    _need(scales, "scales", torch.float16, 2)
+    _need(qzeros, "qzeros", torch.int32, 2)
+    _need(out, "out", torch.float16, 2)
+    K, N, G = _awq_shapes(qweight, scales, qzeros)
+    M = input.shape[0]
+    if input.shape[1] != K or tuple(out.shape) != (M, N):
+        raise ValueError(f"input {tuple(input.shape)} / out {tuple(out.shape)} do not fit K={K}, N={N}")
+    if M == 0:
+        return out
+    split = 0 if force_split_k is None else max(0, min(int(force_split_k), 64))
+    st = _lib.load().awqmi_gemm_f16_noalloc(input.data_ptr(), qweight.data_ptr(), scales.data_ptr(),
+                                            qzeros.data_ptr(), out.data_ptr(), M, K, N, G, split,
+                                            _stream_ptr(input.device))
+    _lib.check(st, "awq_gemm_noalloc")
+    return out
+
+
 def reset_workspace(device=None) -> None:
     """Zeroes the arrival counters of this (device, current stream)'s workspace.  Only needed
     after something cut a call short (a failed or aborted launch): calls that run to completion

@@ -35,8 +35,8 @@ def test_library_exports_every_declared_symbol(lib):
 
 
 def test_status_strings(lib):
-    seen = {lib.awqmi_status_string(i).decode() for i in range(8)}
-    assert len(seen) == 8 and "ok" in seen
+    seen = {lib.awqmi_status_string(i).decode() for i in range(9)}
+    assert len(seen) == 9 and "ok" in seen
     assert lib.awqmi_status_string(99).decode() == "unknown status"
 
 
