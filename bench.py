@@ -29,12 +29,32 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
-# HBM bytes per awq_gemv launch averaged over the decode sweep, from two rocprofv3 --pmc runs
-# (FETCH_SIZE, WRITE_SIZE) of `bench.py --pmc-target decode`, each scaled by what the same
-# counter reads for a 256 MiB device copy; the runs are summarised in
-# profiles/awq_gemv_kernel_decode_sweep_pmc_hbm_traffic.md.  Counters cannot be read while
-# timing, so the figure is carried here and is only valid for the default split-K choice.
-DECODE_SWEEP_TRAFFIC_BYTES = 119090227
+TRAFFIC_PROFILE = os.path.join("profiles", "awq_gemv_kernel_decode_sweep_pmc_hbm_traffic.md")
+
+
+def decode_sweep_traffic(lib, layers, G):
+    """HBM bytes per awq_gemv launch averaged over the decode sweep, as two rocprofv3 --pmc runs
+    (FETCH_SIZE, WRITE_SIZE; counters cannot be read while timing) of `bench.py --pmc-target
+    decode` measured them.  The tracked summary of those runs carries the figure together with
+    the library version and the split-K factors it was measured with; it is only reported when
+    both still describe the library that is running, otherwise None."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
+    except OSError:
+        return None
+    m_bytes = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", text, re.M)
+    m_ver = re.search(r"^library_version:\s*(\d+)", text, re.M)
+    m_split = re.search(r"^split_k:\s*(.+)$", text, re.M)
+    if not (m_bytes and m_ver and m_split):
+        return None
+    if int(m_ver.group(1)) != lib.awqmi_version():
+        return None
+    want = dict(kv.split("=") for kv in m_split.group(1).split())
+    for name, K, N in layers:
+        if str(lib.awqmi_gemm_auto_split_k(16, K, N, G)) != want.get(name):
+            return None
+    return int(m_bytes.group(1))
 
 
 def log(*a):
@@ -262,8 +282,8 @@ def main():
                   "compute_units": torch.cuda.get_device_properties(dev).multi_processor_count},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": DECODE_SWEEP_TRAFFIC_BYTES if args.split_k == 0 and args.variant < 0 else None,
-                     "traffic_source": "profiles/awq_gemv_kernel_decode_sweep_pmc_hbm_traffic.md",
+                     "traffic": decode_sweep_traffic(lib, layers, G) if args.split_k == 0 and args.variant < 0 else None,
+                     "traffic_source": TRAFFIC_PROFILE,
                      "kernel": "awq_gemv_kernel", "avg_launch_us": round(kern_avg_us, 2),
                      "bytes_per_launch": step_bytes // n_launch},
         "decode_points": points,
@@ -407,20 +427,25 @@ def main():
     # ------------------------------------------------------------------ serving-shaped decoder load (opt-in)
     if not args.no_decoder and not args.sweep_only and args.pmc_target is None:
         from importlib import import_module
-        try:
-            dec = import_module(sba.__name__ + ".decoder")
-            torch.cuda.empty_cache()     # the decoder needs about 25 GB
-            res = dec.run_serving_load(dec.QWEN3_30B_A3B, batch=64, prompt_len=1024, new_tokens=256, device=dev)
-            res["workload"] = ("48-layer Qwen3-30B-A3B-shaped synthetic AWQ decoder, batch 64, random prompts of "
-                               "1024 ids, 256 output tokens, greedy, own minimal driver (no vLLM in this image); "
-                               "attention, norms, embedding and lm_head are stock PyTorch")
-            out["decoder"] = res
-            log(f"[bench] decoder: prefill {res['prefill_s']} s, {res['ms_per_decode_step']} ms/decode step, "
-                f"{res['output_tokens_per_s']} output tok/s")
-            log(import_module(sba.__name__ + ".report").format_serving_result(res))
-        except Exception as e:      # a secondary leg: report and keep the headline result
-            out["decoder"] = {"error": f"{type(e).__name__}: {e}"}
-            log(f"[bench] decoder leg failed: {type(e).__name__}: {e}")
+        # a failure in this leg fails the run: it is the only leg that drives the layer methods
+        # (AWQLinearMethod / AWQMoEMethod .apply) at the serving shapes
+        dec = import_module(sba.__name__ + ".decoder")
+        torch.cuda.empty_cache()     # the decoder needs about 25 GB
+        res = dec.run_serving_load(dec.QWEN3_30B_A3B, batch=64, prompt_len=1024, new_tokens=256, device=dev)
+        res["workload"] = ("48-layer Qwen3-30B-A3B-shaped synthetic AWQ decoder, batch 64, random prompts of "
+                           "1024 ids, 256 output tokens, greedy, own minimal driver (no vLLM in this image); "
+                           "attention, norms, embedding and lm_head are stock PyTorch; after the timed load every "
+                           "AWQ call of the first and last layer (one decode step, one prefill) is compared with "
+                           "the dequantize kernel + library matmul on the same input")
+        out["decoder"] = res
+        log(f"[bench] decoder: prefill {res['prefill_s']} s, {res['ms_per_decode_step']} ms/decode step, "
+            f"{res['output_tokens_per_s']} output tok/s; AWQ ops vs dequantize+matmul: "
+            f"{res['awq_ops_rel_frobenius_max']} over {res['awq_ops_checked']} calls")
+        log(import_module(sba.__name__ + ".report").format_serving_result(res))
+        if not res["awq_ops_checked"] or max(res["awq_ops_rel_frobenius_max"].values()) > 2e-3:
+            log("[bench] ERROR: an AWQ op of the decoder differs from dequantize + matmul beyond 2e-3")
+            print(json.dumps(out))
+            sys.exit(1)
 
     # ------------------------------------------------------------------ CPU baseline leg
     if not args.no_cpu:
@@ -428,24 +453,42 @@ def main():
         ncores = os.cpu_count() or 1
         nthreads = min(ncores, int(os.environ.get("OMP_NUM_THREADS", ncores)))
         torch.set_num_threads(nthreads)
-        # bounded sample: two passes over the 16 calls of one step (about 3.7 GB of operands)
-        sample = [(n, K, N, M) for (n, K, N) in layers for M in Ms] * 2
-        sample_bytes, sample_t = 0, 0.0
+
+        def rel(a, b):
+            a, b = a.float(), b.float()
+            return float((a - b).norm() / b.norm())
+
+        # bounded sample: two passes over the 16 calls of one step (about 3.7 GB of operands);
+        # pass 1 times dequantize + matmul as one call (the baseline figure), pass 2 times the two
+        # halves separately
+        calls = [(n, K, N, M) for (n, K, N) in layers for M in Ms]
         worst = 0.0
         n0, K0, N0 = layers[1]
         awq_ref.cpu_linear_torch(X[n0][1].cpu(), *(t.cpu() for t in W[n0][0]), G)      # warm-up
-        for name, K, N, M in sample:
+        sample_bytes, t_both, t_deq, t_mm = 0, 0.0, 0.0, 0.0
+        cpu_points = []
+        for name, K, N, M in calls:
             qw, sc, qz = (t.cpu() for t in W[name][0])
             xc = X[name][M].cpu()
             t1 = time.perf_counter()
             yc = awq_ref.cpu_linear_torch(xc, qw, sc, qz, G)
-            sample_t += time.perf_counter() - t1
-            sample_bytes += workloads.linear_bytes(M, K, N, G)
+            t2 = time.perf_counter()
+            Wc = awq_ref.cpu_dequantize_torch(qw, sc, qz, G)
+            t3 = time.perf_counter()
+            yc2 = awq_ref.cpu_matmul_torch(xc, Wc)
+            t4 = time.perf_counter()
+            t_both += t2 - t1
+            t_deq += t3 - t2
+            t_mm += t4 - t3
+            nb = workloads.linear_bytes(M, K, N, G)
+            sample_bytes += nb
+            cpu_points.append({"layer": name, "M": M, "cpu_ms": round((t2 - t1) * 1e3, 1),
+                               "cpu_dequant_ms": round((t3 - t2) * 1e3, 1), "cpu_matmul_ms": round((t4 - t3) * 1e3, 1),
+                               "cpu_GBps": round(nb / (t2 - t1) / 1e9, 3)})
             # the same call on the GPU must agree with the CPU path (checker)
-            yg = sba.awq_gemm(X[name][M], *W[name][0], 0).float().cpu()
-            err = float((yg - yc.float()).norm() / yc.float().norm())
-            worst = max(worst, err)
-            del qw, sc, qz, yc
+            yg = sba.awq_gemm(X[name][M], *W[name][0], 0).cpu()
+            worst = max(worst, rel(yg, yc), rel(yg, yc2))
+            del qw, sc, qz, yc, yc2, Wc
         # the CPU-runnable configuration (M=16, K=N=4096, seed 0, drawn on the CPU generator)
         c0 = workloads.config0()
         g0 = c0.to(dev)
@@ -461,33 +504,70 @@ def main():
             evs.append((a, b))
         torch.cuda.synchronize()
         t0s = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)
-        cpu_ts = []
+        cpu_ts, deq_ts, mm_ts = [], [], []
         for _ in range(7):
             t1 = time.perf_counter()
             yc0 = awq_ref.cpu_linear_torch(c0.x, c0.qweight, c0.scales, c0.qzeros, 128)
-            cpu_ts.append(time.perf_counter() - t1)
-        cpu_ts = sorted(cpu_ts[2:])
-        err0 = float((y0.float().cpu() - yc0.float()).norm() / yc0.float().norm())
+            t2 = time.perf_counter()
+            Wc0 = awq_ref.cpu_dequantize_torch(c0.qweight, c0.scales, c0.qzeros, 128)
+            t3 = time.perf_counter()
+            awq_ref.cpu_matmul_torch(c0.x, Wc0)
+            t4 = time.perf_counter()
+            cpu_ts.append(t2 - t1); deq_ts.append(t3 - t2); mm_ts.append(t4 - t3)
+        med = lambda ts: sorted(ts[2:])[len(ts[2:]) // 2]      # two warm-ups, five timed, median
+        err0 = rel(y0.cpu(), yc0)
         out["config0"] = {"workload": "M=16, K=N=4096, group 128, seed 0 (cache-warm: 8.9 MB of weights)",
                           "gpu_us_median": round(t0s[len(t0s) // 2], 2), "gpu_us_p10": round(t0s[5], 2),
                           "gpu_us_p90": round(t0s[45], 2),
-                          "cpu_ms_median": round(cpu_ts[len(cpu_ts) // 2] * 1e3, 2), "cpu_threads": nthreads,
+                          "cpu_ms_median": round(med(cpu_ts) * 1e3, 2),
+                          "cpu_dequant_ms_median": round(med(deq_ts) * 1e3, 2),
+                          "cpu_matmul_ms_median": round(med(mm_ts) * 1e3, 2), "cpu_threads": nthreads,
                           "gpu_vs_cpu_rel_frobenius": round(err0, 6)}
         worst = max(worst, err0)
         # one prefill point on the CPU path (o_proj, M = 512: 69 GFLOP; larger ones take minutes)
-        n0, K0, N0 = layers[1]
         xp = torch.randn((512, K0), generator=torch.Generator().manual_seed(512), dtype=torch.float32).half()
         qw, sc, qz = (t.cpu() for t in W[n0][0])
         t1 = time.perf_counter()
-        ycp = awq_ref.cpu_linear_torch(xp, qw, sc, qz, G)
-        cpu_p = time.perf_counter() - t1
-        ygp = sba.awq_gemm(xp.to(dev), *W[n0][0], 0).float().cpu()
-        errp = float((ygp - ycp.float()).norm() / ycp.float().norm())
+        Wc = awq_ref.cpu_dequantize_torch(qw, sc, qz, G)
+        t2 = time.perf_counter()
+        ycp = awq_ref.cpu_matmul_torch(xp, Wc)
+        t3 = time.perf_counter()
+        ygp = sba.awq_gemm(xp.to(dev), *W[n0][0], 0).cpu()
+        errp = rel(ygp, ycp)
         worst = max(worst, errp)
-        cpu_prefill = {"layer": n0, "M": 512, "cpu_ms": round(cpu_p * 1e3, 1),
-                       "cpu_TFLOPs": round(2.0 * 512 * K0 * N0 / cpu_p / 1e12, 4),
+        cpu_prefill = {"layer": n0, "M": 512, "cpu_ms": round((t3 - t1) * 1e3, 1),
+                       "cpu_dequant_ms": round((t2 - t1) * 1e3, 1), "cpu_matmul_ms": round((t3 - t2) * 1e3, 1),
+                       "cpu_TFLOPs": round(2.0 * 512 * K0 * N0 / (t3 - t1) / 1e12, 4),
                        "gpu_vs_cpu_rel_frobenius": round(errp, 6)}
-        del qw, sc, qz, ycp, ygp
+        del qw, sc, qz, ycp, ygp, Wc
+        # the MoE block at T = 1 and 16 on the CPU path (the experts that are hit are dequantised
+        # and applied to their tokens), against the library's one-call block
+        mq = workloads.QWEN3_MOE
+        H, E, topk, I = mq["hidden"], mq["experts"], mq["topk"], mq["inter"]
+        gm = torch.Generator(device=dev).manual_seed(3)
+        w13 = tuple(torch.stack(t) for t in zip(*[make_weights(H, 2 * I, G, dev, gm) for _ in range(E)]))
+        w2 = tuple(torch.stack(t) for t in zip(*[make_weights(I, H, G, dev, gm) for _ in range(E)]))
+        w13c, w2c = tuple(t.cpu() for t in w13), tuple(t.cpu() for t in w2)
+        cpu_moe = []
+        for T in (1, 16):
+            xm = torch.randn((T, H), device=dev, generator=gm).half()
+            lg = torch.randn((T, E), device=dev, generator=gm)
+            tw, ids = sba.topk_softmax(lg, topk, True)
+            ym = sba.fused_moe_awq(xm, w13, w2, lg, topk, True).cpu()
+            xc, idc, twc = xm.cpu(), ids.cpu().long(), tw.cpu()
+            ts = []
+            for _ in range(4):
+                t1 = time.perf_counter()
+                yc = awq_ref.cpu_moe_torch(xc, w13c, w2c, idc, twc, G)
+                ts.append(time.perf_counter() - t1)
+            tm = sorted(ts[1:])[1]
+            distinct = int(torch.unique(idc).numel())
+            errm = rel(ym, yc)
+            worst = max(worst, errm)
+            cpu_moe.append({"T": T, "distinct_experts": distinct, "cpu_ms": round(tm * 1e3, 1),
+                            "cpu_GBps": round(workloads.moe_bytes(distinct, T, H, I, G) / tm / 1e9, 3),
+                            "gpu_vs_cpu_rel_frobenius": round(errm, 6)})
+        del w13, w2, w13c, w2c
         cpu_model = ""
         try:
             with open("/proc/cpuinfo") as f:
@@ -497,13 +577,17 @@ def main():
                         break
         except OSError:
             pass
-        out["cpu_baseline"] = {"value": round(sample_bytes / sample_t / 1e9, 3), "unit": "GB/s",
+        out["cpu_baseline"] = {"value": round(sample_bytes / t_both / 1e9, 3), "unit": "GB/s",
                                "cores": nthreads, "kind": "port",
-                               "sample": f"two passes over the 16 calls of one step, one PyTorch dequantize+matmul "
-                                         f"call each: {len(sample)} calls, {sample_t:.1f} s total",
-                               "cpu": cpu_model, "prefill_point": cpu_prefill,
+                               "sample": f"the 16 calls of one step, one PyTorch dequantize+matmul call each "
+                                         f"({t_both:.1f} s), then dequantize and matmul of the same calls timed "
+                                         f"separately ({t_deq:.1f} s + {t_mm:.1f} s)",
+                               "cpu": cpu_model, "dequant_s": round(t_deq, 2), "matmul_s": round(t_mm, 2),
+                               "together_s": round(t_both, 2), "points": cpu_points,
+                               "prefill_point": cpu_prefill, "moe_points": cpu_moe,
                                "gpu_vs_cpu_rel_frobenius_max": round(worst, 6)}
-        log(f"[bench] cpu baseline {out['cpu_baseline']['value']} GB/s on {nthreads} threads; "
+        log(f"[bench] cpu baseline {out['cpu_baseline']['value']} GB/s on {nthreads} threads "
+            f"(dequantize {t_deq:.1f} s + matmul {t_mm:.1f} s apart, {t_both:.1f} s as one call); "
             f"GPU vs CPU rel. Frobenius max {worst:.2e}")
         if worst > 2e-3:
             log("[bench] ERROR: GPU result differs from the CPU path beyond 2e-3")

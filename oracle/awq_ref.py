@@ -26,6 +26,9 @@ Parity status per function (what pins it, independent of this file's own formula
   topk_softmax            torch.softmax + torch.topk                             PINNED
   topk_sigmoid            torch.sigmoid + torch.topk of score + bias             PINNED
   moe_forward             per-token brute force from pinned W                    PINNED
+  cpu_dequantize_torch / cpu_linear_torch / cpu_moe_torch (the timed CPU baseline)
+                          same bits as dequantize; gemm / moe_forward to fp32
+                          summation order                                        PINNED
   behavioural choices only an import of vLLM could pin (M threshold between fused GEMM
   and dequant+matmul, sentinel/padding layout of its align kernel, [gate | up] order
   inside w13, where its grouped top-k applies the scaling factor)     PARITY UNPINNED
@@ -177,9 +180,8 @@ def moe_forward(x, w13, w2, topk_ids, topk_w, group: int) -> np.ndarray:
 
 # --------------------------------------------------------------------------- baseline
 
-def cpu_linear_torch(x_t, qweight_t, scales_t, qzeros_t, group: int):
-    """The reference CPU path (M=16, K=N=4096 is its CPU-runnable case): PyTorch dequantize
-    then matmul on the host.  Takes and returns torch CPU tensors."""
+def cpu_dequantize_torch(qweight_t, scales_t, qzeros_t, group: int):
+    """PyTorch dequantize on the host: fp16 [K, N] = fp16((w - z) * s).  Torch CPU tensors."""
     import torch
 
     K = qweight_t.shape[0]
@@ -193,5 +195,37 @@ def cpu_linear_torch(x_t, qweight_t, scales_t, qzeros_t, group: int):
     w = unpack(qweight_t)
     z = unpack(qzeros_t).repeat_interleave(group, dim=0)
     s = scales_t.float().repeat_interleave(group, dim=0)
-    W = ((w - z).float() * s).half()
-    return (x_t.float() @ W.float()).half()
+    return ((w - z).float() * s).half()
+
+
+def cpu_matmul_torch(x_t, W_t):
+    """fp16 [M, N] = fp16(X.float() @ W.float()) on the host."""
+    return (x_t.float() @ W_t.float()).half()
+
+
+def cpu_linear_torch(x_t, qweight_t, scales_t, qzeros_t, group: int):
+    """The reference CPU path (M=16, K=N=4096 is its CPU-runnable case): PyTorch dequantize
+    then matmul on the host.  Takes and returns torch CPU tensors.  Pinned against dequantize /
+    gemm above (same bits for W; the product differs from numpy's only in fp32 summation
+    order)."""
+    return cpu_matmul_torch(x_t, cpu_dequantize_torch(qweight_t, scales_t, qzeros_t, group))
+
+
+def cpu_moe_torch(x_t, w13_t, w2_t, topk_ids_t, topk_w_t, group: int):
+    """The MoE block on the host with PyTorch: every expert that is hit is dequantised once and
+    applied to its tokens (fp16 intermediates where the device path stores fp16, fp32 slot sum).
+    Torch CPU tensors; w13 / w2 are (qweight [E, K, N/8], scales, qzeros) triples."""
+    import torch
+
+    T, H = x_t.shape
+    inter = w2_t[0].shape[1]
+    out = torch.zeros((T, H), dtype=torch.float32)
+    for e in torch.unique(topk_ids_t).tolist():
+        tok, slot = torch.nonzero(topk_ids_t == e, as_tuple=True)
+        W13 = cpu_dequantize_torch(w13_t[0][e], w13_t[1][e], w13_t[2][e], group)
+        W2 = cpu_dequantize_torch(w2_t[0][e], w2_t[1][e], w2_t[2][e], group)
+        h = cpu_matmul_torch(x_t[tok], W13).float()
+        a = (torch.nn.functional.silu(h[:, :inter]) * h[:, inter:]).half()
+        o = ((a.float() @ W2.float()) * topk_w_t[tok, slot][:, None]).half().float()
+        out.index_add_(0, tok, o)
+    return out.half()

@@ -24,7 +24,7 @@ import time
 import torch
 import torch.nn.functional as F
 
-from . import awq
+from . import awq, ops
 
 
 @dataclasses.dataclass
@@ -57,6 +57,48 @@ def _rand_awq(shape_k: int, shape_n: int, group: int, dev, gen, lead=()):
 
 class _Layer(torch.nn.Module):
     pass
+
+
+def reference_linear(sub, x: torch.Tensor) -> torch.Tensor:
+    """x @ W with W from the bit-exact dequantize kernel and a library fp32 matmul: the check
+    that the AWQ GEMM kernels are held against at sizes the CPU oracle does not reach."""
+    W = ops.awq_dequantize(sub.qweight, sub.scales, sub.qzeros).float()
+    return x.float() @ W
+
+
+def reference_moe(ex, h: torch.Tensor, logits: torch.Tensor, topk: int) -> torch.Tensor:
+    """The MoE block expert by expert on dequantised weights (routing from the library's top-k
+    kernel, which has its own exact tests); intermediates rounded to fp16 where the kernels
+    store them."""
+    T, H = h.shape
+    inter = ex.w2_qweight.shape[1]
+    w, ids = ops.topk_softmax(logits.float().contiguous(), topk, True)
+    ref = torch.zeros((T, H), dtype=torch.float32, device=h.device)
+    for e in torch.unique(ids).tolist():
+        tok, slot = torch.nonzero(ids == e, as_tuple=True)
+        W13 = ops.awq_dequantize(ex.w13_qweight[e], ex.w13_scales[e], ex.w13_qzeros[e]).float()
+        W2 = ops.awq_dequantize(ex.w2_qweight[e], ex.w2_scales[e], ex.w2_qzeros[e]).float()
+        g = (h[tok].float() @ W13).half().float()
+        a = (F.silu(g[:, :inter]) * g[:, inter:]).half().float()
+        ref.index_add_(0, tok, ((a @ W2) * w[tok, slot][:, None]).half().float())
+    return ref
+
+
+class AwqOpChecker:
+    """Hook for SyntheticMoEDecoder.checker: compares the output of every AWQ call of the chosen
+    layers with reference_linear / reference_moe on the same input and keeps the worst relative
+    Frobenius error per kind.  Eager passes only (it allocates and reads results back)."""
+
+    def __init__(self, topk: int, layers=None):
+        self.topk, self.layers, self.worst, self.calls = topk, layers, {}, 0
+
+    def __call__(self, kind, layer_index, module, inputs, y):
+        if self.layers is not None and layer_index not in self.layers:
+            return
+        ref = reference_moe(module, inputs[0], inputs[1], self.topk) if kind == "moe" else reference_linear(module, inputs[0])
+        err = float((y.float() - ref).norm() / ref.norm())
+        self.worst[kind] = max(self.worst.get(kind, 0.0), err)
+        self.calls += 1
 
 
 class SyntheticMoEDecoder:
@@ -119,6 +161,9 @@ class SyntheticMoEDecoder:
         self.next_tok = torch.zeros(batch, dtype=torch.int64, device=dev)
         self.last_logits = torch.zeros((batch, cfg.vocab), dtype=torch.float16, device=dev)
         self._graph = None
+        # optional hook(kind, layer_index, module, inputs, output) called after every AWQ op of an
+        # eager pass ("qkv", "o", "moe"); must stay None while a graph is captured
+        self.checker = None
 
     # ------------------------------------------------------------------ pieces
     def _rope(self, x, cos, sin):
@@ -127,14 +172,25 @@ class SyntheticMoEDecoder:
         x1, x2 = x[..., :h], x[..., h:]
         return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin), dim=-1)
 
-    def _moe_block(self, L, h):
+    def _moe_block(self, L, h, li=-1):
         cfg = self.cfg
         logits = (h @ L.router).float()
-        return self.moe.apply(L.experts, h, logits, cfg.topk, True)
+        y = self.moe.apply(L.experts, h, logits, cfg.topk, True)
+        if self.checker is not None:
+            self.checker("moe", li, L.experts, (h, logits), y)
+        return y
 
-    def _qkv(self, L, x):
+    def _o(self, L, a, li=-1):
+        y = self.lin.apply(L.o, a)
+        if self.checker is not None:
+            self.checker("o", li, L.o, (a,), y)
+        return y
+
+    def _qkv(self, L, x, li=-1):
         cfg = self.cfg
         qkv = self.lin.apply(L.qkv, x)
+        if self.checker is not None:
+            self.checker("qkv", li, L.qkv, (x,), qkv)
         q, k, v = qkv.split((cfg.heads * cfg.head_dim, cfg.kv_heads * cfg.head_dim, cfg.kv_heads * cfg.head_dim), dim=-1)
         return q, k, v
 
@@ -156,7 +212,7 @@ class SyntheticMoEDecoder:
             x = self.embed[ids[b0:b1].reshape(-1)]                       # [nb * Lp, H]
             for li, L in enumerate(self.layers):
                 h = F.rms_norm(x, (cfg.hidden,), L.ln1, cfg.eps)
-                q, k, v = self._qkv(L, h)
+                q, k, v = self._qkv(L, h, li)
                 q = F.rms_norm(q.reshape(nb, Lp, cfg.heads, cfg.head_dim), (cfg.head_dim,), L.qn, cfg.eps).transpose(1, 2)
                 k = F.rms_norm(k.reshape(nb, Lp, cfg.kv_heads, cfg.head_dim), (cfg.head_dim,), L.kn, cfg.eps).transpose(1, 2)
                 v = v.reshape(nb, Lp, cfg.kv_heads, cfg.head_dim).transpose(1, 2)
@@ -165,9 +221,9 @@ class SyntheticMoEDecoder:
                 self.vc[li][b0:b1, :, :Lp] = v
                 a = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
                 a = a.transpose(1, 2).reshape(nb * Lp, cfg.heads * cfg.head_dim)
-                x = torch.add(x, self.lin.apply(L.o, a.contiguous()), alpha=self.s_o * self.s_qkv)
+                x = torch.add(x, self._o(L, a.contiguous(), li), alpha=self.s_o * self.s_qkv)
                 h = F.rms_norm(x, (cfg.hidden,), L.ln2, cfg.eps)
-                x = torch.add(x, self._moe_block(L, h), alpha=self.s_moe)
+                x = torch.add(x, self._moe_block(L, h, li), alpha=self.s_moe)
             last = x.reshape(nb, Lp, cfg.hidden)[:, -1]
             logits = F.rms_norm(last, (cfg.hidden,), self.norm_f, cfg.eps) @ self.lm_head
             self.last_logits[b0:b1] = logits
@@ -191,7 +247,7 @@ class SyntheticMoEDecoder:
         x = self.embed.index_select(0, self.tok)
         for li, L in enumerate(self.layers):
             h = F.rms_norm(x, (cfg.hidden,), L.ln1, cfg.eps)
-            q, k, v = self._qkv(L, h)
+            q, k, v = self._qkv(L, h, li)
             q = F.rms_norm(q.reshape(B, cfg.heads, cfg.head_dim), (cfg.head_dim,), L.qn, cfg.eps)
             k = F.rms_norm(k.reshape(B, cfg.kv_heads, cfg.head_dim), (cfg.head_dim,), L.kn, cfg.eps)
             q, k = self._rope(q, cos, sin), self._rope(k, cos, sin)
@@ -201,9 +257,9 @@ class SyntheticMoEDecoder:
             s = torch.matmul(qg, self.kc[li].transpose(2, 3)) * scale + mask     # [B, kv, grp, max_len]
             p = torch.softmax(s.float(), dim=-1).half()
             a = torch.matmul(p, self.vc[li]).reshape(B, cfg.heads * cfg.head_dim)
-            x = torch.add(x, self.lin.apply(L.o, a), alpha=self.s_o * self.s_qkv)
+            x = torch.add(x, self._o(L, a, li), alpha=self.s_o * self.s_qkv)
             h = F.rms_norm(x, (cfg.hidden,), L.ln2, cfg.eps)
-            x = torch.add(x, self._moe_block(L, h), alpha=self.s_moe)
+            x = torch.add(x, self._moe_block(L, h, li), alpha=self.s_moe)
         logits = F.rms_norm(x, (cfg.hidden,), self.norm_f, cfg.eps) @ self.lm_head
         self.last_logits.copy_(logits)
         self.next_tok.copy_(logits.argmax(dim=-1))
@@ -211,6 +267,7 @@ class SyntheticMoEDecoder:
     def capture(self):
         """Capture the decode step in a HIP graph (one warm-up step runs first, on the capture
         stream, so that every workspace the step needs exists before the capture)."""
+        assert self.checker is None, "the checker hook reads results back: eager passes only"
         s = torch.cuda.Stream(self.dev)
         s.wait_stream(torch.cuda.current_stream(self.dev))
         with torch.cuda.stream(s):
@@ -241,7 +298,8 @@ class SyntheticMoEDecoder:
 
 
 def run_serving_load(cfg: DecoderConfig = QWEN3_30B_A3B, batch: int = 64, prompt_len: int = 1024,
-                     new_tokens: int = 256, device="cuda:0", seed: int = 0, use_graph: bool = True) -> dict:
+                     new_tokens: int = 256, device="cuda:0", seed: int = 0, use_graph: bool = True,
+                     verify_prefill: bool = True) -> dict:
     """The fixed-length random-prompt load: prefill `batch` prompts, then `new_tokens - 1`
     decode steps (the first output token comes out of the prefill).  Times both phases."""
     dev = torch.device(device)
@@ -263,6 +321,17 @@ def run_serving_load(cfg: DecoderConfig = QWEN3_30B_A3B, batch: int = 64, prompt
     torch.cuda.synchronize(dev)
     t3 = time.perf_counter()
     out_tokens = batch * new_tokens
+    # correctness of what was just timed: one more decode step (eager) and the prefill once more,
+    # with every AWQ call of the first and last layer compared with the
+    # dequantize-kernel + library-matmul reference on the same inputs
+    chk = AwqOpChecker(cfg.topk, layers={0, cfg.layers - 1})
+    model.checker = chk
+    model.pos.fill_(prompt_len + new_tokens - 1)
+    model._decode_step()
+    if verify_prefill:
+        model.prefill(ids)
+    model.checker = None
+    torch.cuda.synchronize(dev)
     return {
         "batch": batch, "prompt_len": prompt_len, "new_tokens": new_tokens, "layers": cfg.layers,
         "prefill_s": round(t1 - t0, 4), "decode_s": round(t3 - t2, 4),
@@ -272,4 +341,6 @@ def run_serving_load(cfg: DecoderConfig = QWEN3_30B_A3B, batch: int = 64, prompt
         "prefill_tokens_per_s": round(batch * prompt_len / (t1 - t0), 1),
         "hip_graph": bool(use_graph),
         "distinct_last_tokens": int(torch.unique(toks[:, -1]).numel()),
+        "awq_ops_checked": chk.calls,
+        "awq_ops_rel_frobenius_max": {k: round(v, 6) for k, v in chk.worst.items()},
     }

@@ -45,3 +45,25 @@ def test_decode_step_continues_prefill(sba, gpu):
     print(f"[decoder] decode-vs-prefill logits rel_fro={err:.2e}", flush=True)
     assert err <= 2e-2
     assert (a.next_tok == b.tok).float().mean().item() >= 0.75
+
+
+def test_full_width_layer_awq_ops_against_dequant_matmul(sba, gpu):
+    """One Qwen3-30B-A3B-width layer (hidden 2048, 32 / 4 heads of 128, 128 experts, top-8,
+    intermediate 768): an 8192-token prefill pass (64 prompts of 128 tokens in one chunk) and a
+    decode step at batch 64, with the output of every AWQ call (qkv, o, MoE block) compared with
+    the dequantize kernel + library matmul / dense expert evaluation on the same input."""
+    from importlib import import_module
+    dec = import_module(sba.__name__ + ".decoder")
+    cfg = dec.DecoderConfig(layers=1, vocab=4096)
+    m = dec.SyntheticMoEDecoder(cfg, 64, 130, gpu, seed=21)
+    ids = torch.randint(0, cfg.vocab, (64, 128), device=gpu, generator=torch.Generator(device=gpu).manual_seed(22))
+    chk = dec.AwqOpChecker(cfg.topk)
+    m.checker = chk
+    m.prefill(ids, chunk_seqs=64)
+    prefill_worst = dict(chk.worst)
+    assert chk.calls == 3
+    m.decode(1, use_graph=False)
+    assert chk.calls == 6
+    print(f"[decoder full width] prefill {prefill_worst} decode-or-prefill max {chk.worst}", flush=True)
+    assert set(chk.worst) == {"qkv", "o", "moe"}
+    assert max(chk.worst.values()) <= 2e-3

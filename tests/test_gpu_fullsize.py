@@ -1,9 +1,13 @@
-"""Benchmark-size checks (Qwen2.5-72B layer shapes), where the CPU oracle would take minutes:
-the GEMM kernels against the bit-exact dequantize kernel followed by a library matmul, plus
-properties that need no reference (rows independent of M, split-K invariance)."""
+"""Benchmark-size checks (Qwen2.5-72B layer shapes and the Qwen3-30B-A3B attention linears),
+where the CPU oracle would take minutes: the dequantize kernel against the oracle on sampled
+rows of the full-size matrices, then the GEMM kernels against that dequantize kernel followed by
+a library matmul, plus properties that need no reference (rows independent of M, split-K
+invariance)."""
 import numpy as np
 import pytest
 import torch
+
+from oracle import awq_ref
 
 pytestmark = pytest.mark.gpu
 
@@ -48,11 +52,37 @@ def test_decode_sizes_against_dequant_matmul(sba, gpu, name, K, N):
         assert _rel(ys, y16) <= 2e-3
 
 
-@pytest.mark.parametrize("name,K,N,M", [("qkv_proj", 8192, 10240, 512), ("o_proj", 8192, 8192, 2048),
-                                        ("down_proj", 29568, 8192, 512), ("gate_up_proj", 8192, 59136, 2048),
-                                        ("o_proj", 8192, 8192, 8192), ("qkv_proj", 8192, 10240, 100),
-                                        ("down_proj", 29568, 8192, 160)])
+@pytest.mark.parametrize("name,K,N", LAYERS)
+def test_full_size_dequantize_rows_against_the_oracle(sba, gpu, name, K, N):
+    """The full-size tests below use the dequantize kernel as their reference, so the kernel itself
+    is anchored here at those sizes: whole rows of its output (first and last rows of the matrix,
+    both sides of group boundaries near the start, the middle and the end, the grid's last row
+    slab, and a random sample) must equal the oracle's bits.  Whole rows cover every word column,
+    the ragged last column block included."""
+    qw, sc, qz, _ = _weights(K, N, gpu, 1)
+    W = sba.awq_dequantize(qw, sc, qz)
+    G, ngroups = 128, K // 128
+    rows = {0, 1, 15, 16, 127, 128, 129, K - 129, K - 128, K - 17, K - 16, K - 1}
+    for gidx in (ngroups // 2, ngroups - 2):
+        rows |= {gidx * G - 1, gidx * G, gidx * G + 127}
+    rows |= set(np.random.default_rng(K + N).integers(0, K, 48).tolist())
+    rows = sorted(rows)
+    ridx = torch.tensor(rows, device=gpu)
+    gidx = ridx // G
+    # each sampled row as a group of its own for the oracle: its packed words, its group's scales / zeros
+    want = awq_ref.dequantize(qw[ridx].cpu().numpy(), sc[gidx].cpu().numpy(), qz[gidx].cpu().numpy(), 1)
+    got = W[ridx].cpu().numpy()
+    assert got.shape == want.shape == (len(rows), N)
+    bad = np.argwhere(got.view(np.uint16) != want.view(np.uint16))
+    assert bad.size == 0, f"{name}: first mismatches (sample row, column) {bad[:5].tolist()} of rows {rows}"
+
+
+PREFILL_POINTS = [(n, K, N, M) for (n, K, N) in LAYERS for M in (512, 2048, 8192)]
+
+
+@pytest.mark.parametrize("name,K,N,M", PREFILL_POINTS + [("qkv_proj", 8192, 10240, 100), ("down_proj", 29568, 8192, 160)])
 def test_prefill_sizes_against_dequant_matmul(sba, gpu, name, K, N, M):
+    """All twelve (layer, M) points of the prefill sweep and two off-grid row counts."""
     qw, sc, qz, g = _weights(K, N, gpu, 2)
     W = sba.awq_dequantize(qw, sc, qz)
     x = torch.randn((M, K), device=gpu, generator=g).half()
@@ -66,6 +96,21 @@ def test_prefill_sizes_against_dequant_matmul(sba, gpu, name, K, N, M):
     assert worst <= TOL
     y2 = sba.awq_gemm(x, qw, sc, qz, 0)
     assert torch.equal(y, y2)          # deterministic
+
+
+@pytest.mark.parametrize("name,K,N", [("qwen3-30b-a3b qkv", 2048, 5120), ("qwen3-30b-a3b o", 4096, 2048)])
+@pytest.mark.parametrize("M", [1, 16, 64, 8192])
+def test_moe_decoder_attention_linears(sba, gpu, name, K, N, M):
+    """The two dense AWQ linears of the Qwen3-30B-A3B-shaped decoder at its decode batch (64),
+    its prefill pass (8 prompts x 1024 tokens) and the skinny sizes."""
+    qw, sc, qz, g = _weights(K, N, gpu, 4)
+    W = sba.awq_dequantize(qw, sc, qz).float()
+    x = torch.randn((M, K), device=gpu, generator=g).half()
+    y = sba.awq_gemm(x, qw, sc, qz, 0)
+    err = _rel(y, x.float() @ W)
+    print(f"[full {name} M={M}] rel_fro={err:.2e}", flush=True)
+    assert err <= TOL
+    assert torch.equal(y, sba.awq_gemm(x, qw, sc, qz, 0))
 
 
 def test_activations_beyond_4gib_run_as_row_slabs(sba, gpu):

@@ -335,3 +335,30 @@ def test_topk_sigmoid_matches_torch():
     ids2, w2 = awq_ref.topk_sigmoid(logits.numpy(), 5, False)
     assert np.array_equal(ids2, torch.topk(score, 5, dim=-1).indices.numpy().astype(np.int32))
     assert np.allclose(w2, torch.topk(score, 5, dim=-1).values.numpy(), rtol=1e-6)
+
+
+def test_cpu_baseline_functions_against_the_pinned_oracle():
+    """The PyTorch functions that the benchmark times as the CPU baseline (and uses to check GPU
+    results at benchmark sizes): their dequantised weights carry the oracle's bits, and their
+    products equal the oracle's fp32-accumulated ones up to the summation order of the two
+    libraries (one fp16 ulp on a few elements, far inside 2e-3 of the float64 product)."""
+    import torch
+    import server_benchmark_amd as sba
+    c = sba.workloads.config0()                    # M = 16, K = N = 4096, group 128, seed 0
+    x, qw, s, qz = (t.numpy() for t in (c.x, c.qweight, c.scales, c.qzeros))
+    Wt = awq_ref.cpu_dequantize_torch(c.qweight, c.scales, c.qzeros, 128).numpy()
+    assert np.array_equal(Wt.view(np.uint16), awq_ref.dequantize(qw, s, qz, 128).view(np.uint16))
+    yt = awq_ref.cpu_linear_torch(c.x, c.qweight, c.scales, c.qzeros, 128).numpy()
+    yn = awq_ref.gemm(x, qw, s, qz, 128, acc=np.float32)
+    # one fp16 ulp apart at most, plus the fp32 summation-order noise where the sum cancels
+    d = np.abs(yt.astype(np.float64) - yn.astype(np.float64))
+    assert np.all(d <= 2.0 ** -10 * np.abs(yn.astype(np.float64)) + 1e-4)
+    assert (yt.view(np.uint16) == yn.view(np.uint16)).mean() >= 0.99
+    assert awq_ref.rel_frobenius(yt, awq_ref.gemm_wide(x, qw, s, qz, 128)) <= 4e-4
+    # group = -1 (one group over K) and the MoE form against the per-token brute force
+    m = sba.workloads.make_moe_case(5, 256, 8, 2, 128, 128, seed=9)
+    ids, tw = awq_ref.topk_softmax(m.logits.numpy(), 2, True)
+    want = awq_ref.moe_forward(m.x.numpy(), tuple(a.numpy() for a in m.w13), tuple(a.numpy() for a in m.w2),
+                               ids, tw, 128)
+    got = awq_ref.cpu_moe_torch(m.x, m.w13, m.w2, torch.from_numpy(ids), torch.from_numpy(tw), 128).numpy()
+    assert awq_ref.rel_frobenius(got, want) <= 1e-3
