@@ -93,6 +93,9 @@ def main():
                          "decode sweep twice (direct launches) plus four 256 MiB device copies "
                          "(calibration of FETCH_SIZE / WRITE_SIZE).  prefill: awq_gemm at o_proj, "
                          "M=8192, three times.  moe: the Qwen3-30B-A3B MoE block at T=512, five times")
+    ap.add_argument("--pmc-data", choices=("random", "const"), default="random",
+                    help="with --pmc-target prefill: random operands (the benchmark's data) or the same value in "
+                         "every weight, zero point, scale and activation (no operand bit toggles in the matrix pipe)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -152,6 +155,9 @@ def main():
         name, K, N = layers[1]
         qw, sc, qz = W[name][0]
         xp = torch.randn((8192, K), device=dev, generator=gen).to(torch.float16)
+        if args.pmc_data == "const":
+            qw, sc, qz = torch.full_like(qw, 0x77777777), torch.full_like(sc, 0.01), torch.full_like(qz, 0x33333333)
+            xp.fill_(1.0)
         yp = torch.empty((8192, N), dtype=torch.float16, device=dev)
         for _ in range(3):
             st = lib.awqmi_gemm_f16(xp.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), yp.data_ptr(),
@@ -160,7 +166,7 @@ def main():
             assert st == 0
         torch.cuda.synchronize()
         log(f"[bench] pmc target: 3 x awq_gemm {name} M=8192 K={K} N={N} "
-            f"({workloads.linear_flops(8192, K, N)} flops each)")
+            f"({workloads.linear_flops(8192, K, N)} flops each), {args.pmc_data} operands")
         return
     if args.pmc_target == "moe":
         mq = workloads.QWEN3_MOE
