@@ -97,7 +97,7 @@ struct WordVec<2> {
 // operand costs one v_perm_b32 + one v_and_b32 per four weights and no conversion.
 // Per quantisation group and 16-column tile the wave keeps accg = 2^-e * sum_k x_k (w_k - z):
 // the sum over w comes from the unpacked nibbles, the zero point from one more MFMA whose A
-// operand holds this lane's sum of x over the group (split into three fp16 pieces) and whose
+// operand holds this lane's sum of x over the group (split into four fp16 pieces) and whose
 // B operand holds -z * 2^-e.  At the end of the group acc += s * accg (fp32, one v_fma_mix per
 // element); the factor 2^e is applied once when the wave leaves the loop.
 //
@@ -240,34 +240,51 @@ struct GemvWave {
          : b == 2 ? byte_pair<2>(zw, zw) : byte_pair<3>(zw, zw);
   }
 
-  // end of a group: zero-point MFMA, then acc += s * accg
-  __device__ __forceinline__ void flush() {
+  // Zero-point MFMA: accg -= 2^-e * z * (this lane's sum of x since the last call).  The sum goes
+  // in as four fp16 pieces, each clamped to the fp16 range before it is taken off the rest: a
+  // sum below 65504 in magnitude splits as before (first piece = the rounded sum, the others its
+  // residuals, 33+ significant bits), and larger sums (large-mean or outlier activations) stay
+  // exact up to 4 x 65504 instead of turning into inf.  A lane adds at most 32 activations
+  // between two calls (G = 128 * i calls this once per 128-row chunk for that reason).
+  __device__ __forceinline__ void flush_zero() {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      // xsum as three fp16 pieces (33 significant bits) in k-slots 0..2 against -z there
-      const half_t x0 = (half_t)xsum[mb];
-      const float r1 = xsum[mb] - (float)x0;
-      const half_t x1 = (half_t)r1;
-      const half_t x2 = (half_t)(r1 - (float)x1);
-      const h2 xp01 = {x0, x1}, xp2 = {x2, (half_t)0.f};
-      // (the 16-deep MFMA: its four k-slots per lane hold the three pieces and a zero, so neither
-      // operand needs zero padding registers)
-      const h4 az = __builtin_bit_cast(h4, u2v{as_u32(xp01), as_u32(xp2)});
+      constexpr float HMAX = 65504.f;
+      float r = xsum[mb];
+      const half_t x0 = (half_t)__builtin_fmaxf(-HMAX, __builtin_fminf(HMAX, r));
+      r -= (float)x0;
+      const half_t x1 = (half_t)__builtin_fmaxf(-HMAX, __builtin_fminf(HMAX, r));
+      r -= (float)x1;
+      const half_t x2 = (half_t)__builtin_fmaxf(-HMAX, __builtin_fminf(HMAX, r));
+      r -= (float)x2;
+      const half_t x3 = (half_t)__builtin_fmaxf(-HMAX, __builtin_fminf(HMAX, r));
+      const h2 xp01 = {x0, x1}, xp23 = {x2, x3};
+      // (the 16-deep MFMA: its four k-slots per lane hold the four pieces, so neither operand
+      // needs zero padding registers)
+      const h4 az = __builtin_bit_cast(h4, u2v{as_u32(xp01), as_u32(xp23)});
 #pragma unroll
       for (int w = 0; w < WPL; ++w) {
         const uint32_t zw = WordVec<WPL>::get(zcur, w);
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
-          // B operand word of the zero-point MFMA: (-z, -z) * 2^-e in k-slots 0, 1 and -z in 2
+          // B operand word of the zero-point MFMA: -z * 2^-e in all four k-slots
           const uint32_t t = zbyte(zw, b);
           const uint32_t zlo = t | 0x80008000u, zhi = (t & nm.hi) | 0x80008000u;
           const int t0 = w * 8 + 2 * b;
           accg[mb][t0] = __builtin_amdgcn_mfma_f32_16x16x16f16(
-              az, __builtin_bit_cast(h4, u2v{zlo, zlo & 0x0000FFFFu}), accg[mb][t0], 0, 0, 0);
+              az, __builtin_bit_cast(h4, u2v{zlo, zlo}), accg[mb][t0], 0, 0, 0);
           accg[mb][t0 + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(
-              az, __builtin_bit_cast(h4, u2v{zhi, zhi & 0x0000FFFFu}), accg[mb][t0 + 1], 0, 0, 0);
+              az, __builtin_bit_cast(h4, u2v{zhi, zhi}), accg[mb][t0 + 1], 0, 0, 0);
         }
       }
+      if (GMODE == 3) xsum[mb] = 0.f;
+    }
+  }
+
+  // end of a group: acc += s * accg
+  __device__ __forceinline__ void flush_scale() {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
       for (int w = 0; w < WPL; ++w) {
         const h8 sv = as_h8(scur[w]);
@@ -282,6 +299,11 @@ struct GemvWave {
         }
       }
     }
+  }
+
+  __device__ __forceinline__ void flush() {
+    flush_zero();
+    flush_scale();
   }
 
   // one aligned 128-row chunk (four ring slots); REFILL: chunk c + 1 belongs to this wave too.
@@ -326,7 +348,8 @@ struct GemvWave {
     }
     if (GMODE == 3) {
       const int cpg = kspg >> 2;
-      if (c + 1 == c_end || (c + 1) % cpg == 0) flush();
+      flush_zero();
+      if (c + 1 == c_end || (c + 1) % cpg == 0) flush_scale();
     }
   }
 

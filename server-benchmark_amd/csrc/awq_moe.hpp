@@ -85,6 +85,16 @@ __device__ __forceinline__ void moe_topk_token(const float* __restrict__ logits,
       const unsigned long long b = __ballot(open[i] && v[i] == best);
       if (b) bidx = 64 * i + __builtin_ctzll(b);
     }
+    if (bidx == E) {
+      // only NaN keys are left (fmaxf skipped them, nothing equals `best`): take the lowest
+      // expert that is still open, so that every id stays inside [0, E) and every slot gets its
+      // rows written; the weight computed below is NaN and carries the bad logit forward
+#pragma unroll
+      for (int i = PER - 1; i >= 0; --i) {
+        const unsigned long long b = __ballot(open[i]);
+        if (b) bidx = 64 * i + __builtin_ctzll(b);
+      }
+    }
     float bsc = 0.f;
     if (SIGMOID) {
 #pragma unroll
@@ -92,7 +102,14 @@ __device__ __forceinline__ void moe_topk_token(const float* __restrict__ logits,
         if ((bidx >> 6) == i)
           bsc = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sc[i]), bidx & 63));
     }
-    const float pw = SIGMOID ? bsc : __expf(best - mx) / sum;
+    float bkey = best;                               // the winner's own key (NaN when only NaN keys are left)
+    if (!SIGMOID) {
+#pragma unroll
+      for (int i = 0; i < PER; ++i)
+        if ((bidx >> 6) == i)
+          bkey = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[i]), bidx & 63));
+    }
+    const float pw = SIGMOID ? bsc : __expf(bkey - mx) / sum;
     sel_sum += pw;
     if (lane == it) { my_w = pw; my_id = bidx; }
 #pragma unroll

@@ -28,6 +28,42 @@ def test_topk_softmax(sba, gpu, T, E, topk):
     assert ids.cpu().tolist() == [list(range(topk))] * 2
 
 
+@pytest.mark.parametrize("scoring", ["softmax", "sigmoid"])
+def test_topk_with_nan_and_infinite_logits_keeps_ids_in_range(sba, gpu, scoring):
+    """Rows with fewer than top-k usable logits: NaN keys lose against every number and are then
+    taken in expert order (the oracle's stable argsort puts them last the same way), -inf keys
+    tie towards the lowest id.  Every id must be a distinct expert inside [0, E) - an id of E
+    would leave that slot's rows unwritten - and the block built on such routing must still
+    write every output row.  (How vLLM's own routing kernel orders NaN keys is not pinned by
+    anything available here; the weights of such rows are NaN on both sides.)"""
+    E, topk = 128, 8
+    lg = torch.randn((6, E), generator=torch.Generator().manual_seed(1))
+    lg[0, 5:] = float("nan")                 # five numbers, the rest NaN
+    lg[1, :] = float("nan")                  # nothing usable
+    lg[2, :] = float("-inf")                 # all tied at -inf
+    lg[3, 3:] = float("-inf")                # three numbers, the rest -inf
+    lg[4, ::2] = float("nan")                # every other one NaN
+    if scoring == "softmax":
+        w, ids = sba.topk_softmax(lg.to(gpu), topk, True)
+        rid, rw = awq_ref.topk_softmax(lg.numpy(), topk, True)
+    else:
+        w, ids = sba.topk_route(lg.to(gpu), topk, True, "sigmoid")
+        rid, rw = awq_ref.topk_sigmoid(lg.numpy(), topk, True)
+    ids, w = ids.cpu().numpy(), w.cpu().numpy()
+    assert ids.min() >= 0 and ids.max() < E
+    assert all(len(set(r.tolist())) == topk for r in ids)
+    assert np.array_equal(ids, rid)
+    assert np.allclose(w, rw, rtol=2e-5, atol=1e-8, equal_nan=True)
+    assert np.isfinite(w[5]).all() and np.isfinite(w[3]).all() and np.isnan(w[[0, 1]]).all()
+    if scoring == "softmax":
+        assert np.isnan(w[[2, 4]]).all()
+        c = sba.workloads.make_moe_case(6, 256, E, topk, 128, 128, seed=4).to(gpu)
+        y = sba.fused_moe_awq(c.x, c.w13, c.w2, lg.to(gpu), topk, True)
+        torch.cuda.synchronize()
+        assert torch.isfinite(y[5]).all() and torch.isfinite(y[3]).all()      # rows with usable routing
+        assert torch.isnan(y[[0, 1, 2, 4]]).all()      # NaN weights reach every element: no row is stale
+
+
 @pytest.mark.parametrize("T,E,topk,tile", [(1, 128, 8, 16), (16, 128, 8, 16), (512, 128, 8, 16), (7, 4, 2, 4),
                                            (1000, 8, 2, 16), (64, 1024, 4, 16), (3, 5, 1, 1), (4096, 128, 8, 16)])
 def test_moe_align_equals_oracle(sba, gpu, T, E, topk, tile):

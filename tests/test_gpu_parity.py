@@ -184,6 +184,42 @@ def test_gemm_one_hot_is_exact_and_zero_weights(sba, gpu):
     assert not sba.awq_gemm(*_dev(gpu, xl, awq_ref.pack_awq(zfull), s, qz), 0).cpu().numpy().any()
 
 
+@pytest.mark.parametrize("K,N,G,M", [(4096, 256, -1, 5), (4096, 512, 128, 16), (1024, 264, 1024, 3), (2048, 256, 256, 32)])
+def test_gemm_decode_large_mean_and_outlier_activations(sba, gpu, K, N, G, M):
+    """The skinny kernel takes the zero point out through a lane's running sum of x fed to the
+    matrix core as fp16 pieces: activations with a large mean (sums of tens of thousands per lane
+    and group, more with one group over all of K) or massive outliers must neither overflow that
+    sum nor cost accuracy.  Checked against the float64 product with a max-abs bound next to the
+    relative Frobenius one."""
+    rng = np.random.default_rng(K + N + M)
+    g = K if G <= 0 else G
+    w = rng.integers(0, 16, (K, N))
+    z = rng.integers(0, 16, (K // g, N))
+    s = (rng.random((K // g, N)) * 0.019 + 0.001).astype(np.float16)
+    qw, qz = awq_ref.pack_awq(w), awq_ref.pack_awq(z)
+    cases = {
+        "mean 100": rng.normal(100.0, 1.0, (M, K)),
+        "mean -3000": rng.normal(-3000.0, 10.0, (M, K)),
+        "outliers": rng.normal(0.0, 1.0, (M, K)),
+    }
+    cases["outliers"][:, rng.integers(0, K, 6)] = 30000.0
+    cases["outliers"][:, rng.integers(0, K, 6)] = -28000.0
+    for name, x in cases.items():
+        x = x.astype(np.float16)
+        ref = awq_ref.gemm_wide(x, qw, s, qz, g)
+        if np.abs(ref).max() >= 60000:      # keep the true result inside fp16
+            x = (x.astype(np.float32) * (30000.0 / np.abs(ref).max())).astype(np.float16)
+            ref = awq_ref.gemm_wide(x, qw, s, qz, g)
+        y = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), 0).cpu().numpy().astype(np.float64)
+        assert np.isfinite(y).all(), name
+        err = awq_ref.rel_frobenius(y, ref)
+        maxabs = float(np.abs(y - ref).max())
+        scale = float(np.abs(ref).max())
+        print(f"[gemm {name} M={M} K={K} N={N} G={g}] rel_fro={err:.2e} max_abs={maxabs:.3e} of {scale:.3e}", flush=True)
+        assert err <= TOL, name
+        assert maxabs <= 2e-3 * scale, name
+
+
 def test_gemm_config0(sba, gpu):
     c = sba.workloads.config0()
     x, qw, s, qz = (t.numpy() for t in (c.x, c.qweight, c.scales, c.qzeros))
