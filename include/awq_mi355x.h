@@ -41,7 +41,7 @@ typedef enum awqmi_status {
   AWQMI_SCRATCH_LIMIT = 8        /* awqmi_gemm_f16_noalloc: needs > AWQMI_STATIC_SCRATCH_BYTES */
 } awqmi_status;
 
-#define AWQMI_VERSION 100        /* major*10000 + minor*100 + patch */
+#define AWQMI_VERSION 200        /* major*10000 + minor*100 + patch */
 #define AWQMI_MOE_TILE_M 16      /* default rows per sorted-token block (32 also accepted)  */
 #define AWQMI_MAX_SPLIT_K 64
 #define AWQMI_MAX_EXPERTS 1024

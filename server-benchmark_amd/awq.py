@@ -203,6 +203,8 @@ class AWQMoEMethod:
             raise NotImplementedError("a score-correction bias is only implemented for sigmoid scoring")
         if activation != "silu":
             raise NotImplementedError(f"activation {activation!r} is not implemented (silu only)")
+        if unused.get("apply_router_weight_on_input"):
+            raise NotImplementedError("routing weights applied to the expert input are not implemented")
         if expert_map is not None or (global_num_experts not in (-1, layer.w13_qweight.shape[0])):
             raise NotImplementedError("expert parallelism (expert_map / global_num_experts) is not implemented")
         shape = x.shape

@@ -1,10 +1,13 @@
-"""Import alias: the package directory is `server-benchmark_amd/`, which is not a Python
-identifier; `import server_benchmark_amd` resolves to it."""
-import importlib
+"""Import name of the package: its directory is `server-benchmark_amd/`, which is not a Python
+identifier, so this module loads that directory's `__init__.py` as the package
+`server_benchmark_amd` (submodules resolve inside the directory, under this one name)."""
+import importlib.util
 import os
 import sys
 
-_root = os.path.dirname(os.path.abspath(__file__))
-if _root not in sys.path:
-    sys.path.insert(0, _root)
-sys.modules[__name__] = importlib.import_module("server-benchmark_amd")
+_pkg_dir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "server-benchmark_amd")
+_spec = importlib.util.spec_from_file_location(__name__, os.path.join(_pkg_dir, "__init__.py"),
+                                               submodule_search_locations=[_pkg_dir])
+_pkg = importlib.util.module_from_spec(_spec)
+sys.modules[__name__] = _pkg
+_spec.loader.exec_module(_pkg)

@@ -126,3 +126,69 @@ def test_gpu_count_and_nginx_conf(deploy):
     conf = deploy.nginx_conf(3)
     assert conf.count("server vllm_") == 3 and "least_conn;" in conf and "listen 8080;" in conf
     assert "proxy_buffering off;" in conf and conf.count("{") == conf.count("}")
+
+
+def test_cli_writes_the_recorded_stack(deploy, tmp_path, monkeypatch):
+    """The command line the harness's step script uses for its own generator (reference
+    benchmarks/3_vllm_benchmark.sh:46-63, flags of utils/generate_compose.py:261-332), pointed
+    at this file: the files it writes must carry the recorded stack's vendor-independent parts
+    and nginx.conf, and the reference's messages."""
+    out, conf = tmp_path / "docker-compose.vllm.yml", tmp_path / "nginx.vllm.conf"
+    monkeypatch.setattr(deploy, "total_rocm_gpus", lambda: 4)
+    argv = ["--num-instances", "4", "--tensor-parallel-size", "1", "--pipeline-parallel-size", "1",
+            "--container-name", "vllm_benchmark_container", "--model-path", f"/hf_models/{MODEL}",
+            "--model-name", MODEL, "--hf-directory", "/hf_models", "--hf-token", "",
+            "--extra-args", "--max-model-len 8192", "--output", str(out), "--nginx-conf-output", str(conf)]
+    assert deploy.main(argv) == 0
+    want = yaml.safe_load(GOLD.read_text())["services"]
+    got = yaml.safe_load(out.read_text())["services"]
+    assert list(got) == list(want)
+    for i in range(4):
+        g, w = got[f"vllm_{i}"], want[f"vllm_{i}"]
+        for key in ("container_name", "ports", "shm_size", "ipc", "healthcheck"):
+            assert g[key] == w[key], key
+        assert g["command"].split() == w["command"].split()
+        assert f"HIP_VISIBLE_DEVICES={i}" in g["environment"]
+    assert got["nginx"]["volumes"] == [f"{conf}:/etc/nginx/nginx.conf:ro"]       # absolute path, as docker wants it
+    assert got["nginx"]["depends_on"] == want["nginx"]["depends_on"]
+    assert conf.read_text() == deploy.nginx_conf(4)
+    # several instances without a place for nginx.conf: the reference's error, exit status 1
+    assert deploy.main(argv[:-2]) == 1
+    # one instance that takes every GPU of the host sees all devices; with the library mounted the
+    # server gets the plugin's path
+    one = tmp_path / "one.yml"
+    monkeypatch.setattr(deploy, "total_rocm_gpus", lambda: 8)
+    assert deploy.main(["--num-instances", "1", "--tensor-parallel-size", "8", "--container-name", "c",
+                        "--model-path", "/m", "--model-name", "m", "--hf-directory", "/hf", "-o", str(one),
+                        "--library-dir", "/srv/awq"]) == 0
+    svc = yaml.safe_load(one.read_text())["services"]["vllm_0"]
+    assert not any(e.startswith("HIP_VISIBLE_DEVICES") for e in svc["environment"])
+    assert "/srv/awq:/opt/awq_mi355x:ro" in svc["volumes"] and "PYTHONPATH=/opt/awq_mi355x" in svc["environment"]
+    with pytest.raises(SystemExit):
+        deploy.main(["--num-instances", "1"])
+
+
+def test_gpu_count_runs_rocminfo_and_system_info_section(deploy):
+    import subprocess
+    text = "\n".join(["Agent 1", "  Device Type:             CPU", "Agent 2", "  Device Type:             GPU",
+                      "Agent 3", "  Device Type:             GPU"])
+    calls = []
+
+    def runner(cmd, **kw):
+        calls.append(cmd)
+        assert kw.get("check") and kw.get("capture_output") and kw.get("text")
+        if cmd[0] == "rocminfo":
+            return subprocess.CompletedProcess(cmd, 0, stdout=text, stderr="")
+        if cmd == ["rocm-smi"]:
+            return subprocess.CompletedProcess(cmd, 0, stdout="GPU  Temp  Power\n0    35c   140W\n", stderr="")
+        raise subprocess.CalledProcessError(2, cmd)
+
+    def absent(cmd, **kw):
+        raise FileNotFoundError(cmd[0])
+
+    assert deploy.total_rocm_gpus(runner) == 2 and calls == [["rocminfo"]]
+    assert deploy.total_rocm_gpus(absent) == 0                 # no tool: 0 GPUs, as the harness counts
+    sec = deploy.system_info_gpu_section(runner)
+    assert sec.startswith("=== GPU INFORMATION ===\n")
+    assert "=== ROCM-SMI FULL OUTPUT ===\nGPU  Temp  Power" in sec and "=== ROCMINFO (2 GPU agents) ===" in sec
+    assert deploy.system_info_gpu_section(absent) == "=== GPU INFORMATION ===\nNo GPU information available\n"

@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol(lib):
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
     assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
-    assert lib.awqmi_version() == 100
+    assert lib.awqmi_version() == 200
 
 
 def test_status_strings(lib):
@@ -300,23 +300,161 @@ def test_workload_pack_matches_oracle(sba):
     assert np.array_equal(sba.workloads.pack_int4_awq(v).numpy(), awq_ref.pack_awq(v.numpy()))
 
 
+def _fake_vllm(monkeypatch, with_registry=True):
+    """Stand-in modules with the attribute names the plugin relies on."""
+    import sys, types
+    for name in [m for m in sys.modules if m == "vllm" or m.startswith("vllm.")]:
+        monkeypatch.delitem(sys.modules, name, raising=False)
+    mods = {}
+
+    def mod(name, **attrs):
+        m = types.ModuleType(name)
+        m.__path__ = []
+        for k, v in attrs.items():
+            setattr(m, k, v)
+        monkeypatch.setitem(sys.modules, name, m)
+        mods[name] = m
+        return m
+
+    old = lambda *a, **k: (_ for _ in ()).throw(AssertionError("vLLM's own op was called"))
+    mod("vllm")
+    mod("vllm._custom_ops", awq_gemm=old, awq_dequantize=old)
+    mod("vllm.envs", VLLM_USE_TRITON_AWQ=True)
+    if with_registry:
+        class QuantizationConfig:                      # vLLM's base class
+            def __init__(self):
+                self.packed_modules_mapping = {}
+
+        class FusedMoE(torch.nn.Module):
+            pass
+
+        class LinearBase(torch.nn.Module):
+            pass
+
+        mod("vllm.model_executor")
+        mod("vllm.model_executor.layers")
+        mod("vllm.model_executor.layers.quantization", QUANTIZATION_METHODS=["awq", "gptq", "awq_marlin"],
+            _CUSTOMIZED_METHOD_TO_QUANT_CONFIG={})
+        mod("vllm.model_executor.layers.quantization.base_config", QuantizationConfig=QuantizationConfig)
+        mod("vllm.model_executor.layers.fused_moe", FusedMoE=FusedMoE)
+        mod("vllm.model_executor.layers.linear", LinearBase=LinearBase)
+    return mods
+
+
 def test_vllm_plugin_rebinds_ops(sba, monkeypatch):
     """Against a stand-in `vllm._custom_ops`: both ops are rebound to this package's functions
-    (same argument order as vLLM's); without vLLM the plugin raises ImportError."""
-    import importlib, inspect, sys, types
+    (same argument order as vLLM's); without vLLM the plugin raises ImportError; without the
+    quantisation registry the ops are still rebound, with a warning."""
+    import importlib, inspect, sys
     plugin = importlib.import_module(sba.__name__ + ".vllm_plugin")
-    monkeypatch.delitem(sys.modules, "vllm", raising=False)
-    monkeypatch.delitem(sys.modules, "vllm._custom_ops", raising=False)
+    for name in [m for m in sys.modules if m == "vllm" or m.startswith("vllm.")]:
+        monkeypatch.delitem(sys.modules, name, raising=False)
     with pytest.raises(ImportError):
         plugin.register()
-    vllm = types.ModuleType("vllm")
-    vllm.__path__ = []
-    ops_mod = types.ModuleType("vllm._custom_ops")
-    ops_mod.awq_gemm = ops_mod.awq_dequantize = lambda *a: (_ for _ in ()).throw(AssertionError("old op"))
-    monkeypatch.setitem(sys.modules, "vllm", vllm)
-    monkeypatch.setitem(sys.modules, "vllm._custom_ops", ops_mod)
-    assert plugin.register() == ["awq_dequantize", "awq_gemm"]
+    mods = _fake_vllm(monkeypatch, with_registry=False)
+    ops_mod = mods["vllm._custom_ops"]
+    with pytest.warns(UserWarning):
+        assert plugin.register() == ["awq_dequantize", "awq_gemm"]
     assert ops_mod.awq_gemm is sba.awq_gemm and ops_mod.awq_dequantize is sba.awq_dequantize
     assert list(inspect.signature(ops_mod.awq_gemm).parameters)[:5] == \
         ["input", "qweight", "scales", "qzeros", "split_k_iters"]
     assert list(inspect.signature(ops_mod.awq_dequantize).parameters)[:3] == ["qweight", "scales", "zeros"]
+    assert mods["vllm.envs"].VLLM_USE_TRITON_AWQ is False
+
+
+def test_vllm_plugin_registers_the_awq_method_for_linear_and_moe_layers(sba, monkeypatch):
+    """The harness passes no --quantization flag, so the method must win by the checkpoint's
+    name: after register() vLLM's registry maps `awq` to this package's config, which hands
+    AWQMoEMethod to FusedMoE layers and AWQLinearMethod to linear layers, and the MoE method's
+    apply (called with vLLM's keyword surface) reaches ops.fused_moe_awq."""
+    import importlib
+    plugin = importlib.import_module(sba.__name__ + ".vllm_plugin")
+    ops = importlib.import_module(sba.__name__ + ".ops")
+    mods = _fake_vllm(monkeypatch)
+    assert plugin.register() == ["awq_dequantize", "awq_gemm", "quantization:awq"]
+    quant = mods["vllm.model_executor.layers.quantization"]
+    cls = quant._CUSTOMIZED_METHOD_TO_QUANT_CONFIG["awq"]
+    assert quant.QUANTIZATION_METHODS.count("awq") == 1
+    assert issubclass(cls, sba.AWQConfig)
+    assert issubclass(cls, mods["vllm.model_executor.layers.quantization.base_config"].QuantizationConfig)
+    assert cls.get_name() == "awq"
+    assert cls.override_quantization_method({"quant_method": "awq", "bits": 4}, None) == "awq"
+    assert cls.override_quantization_method({"quant_method": "gptq"}, None) is None
+    cfg = cls.from_config({"quant_method": "awq", "bits": 4, "group_size": 128, "zero_point": True,
+                           "modules_to_not_convert": ["mlp.gate."]})
+    assert cfg.packed_modules_mapping == {} and cfg.group_size == 128       # both base classes initialised
+    moe_layer = mods["vllm.model_executor.layers.fused_moe"].FusedMoE()
+    lin_layer = mods["vllm.model_executor.layers.linear"].LinearBase()
+    assert isinstance(cfg.get_quant_method(lin_layer, "model.layers.0.self_attn.qkv_proj"), sba.AWQLinearMethod)
+    assert cfg.get_quant_method(lin_layer, "model.layers.0.mlp.gate.") is None        # the router stays fp16
+    assert cfg.get_quant_method(torch.nn.LayerNorm(4), "model.norm") is None
+    method = cfg.get_quant_method(moe_layer, "model.layers.0.mlp.experts")
+    assert isinstance(method, sba.AWQMoEMethod)
+    method.create_weights(moe_layer, 4, 256, 128, torch.float16)
+    seen = {}
+
+    def fake_fused(hidden, w13, w2, logits, topk, renorm, **kw):
+        seen.update(topk=topk, renorm=renorm, w13=w13[0].shape, w2=w2[0].shape, kw=kw)
+        return torch.zeros_like(hidden)
+
+    monkeypatch.setattr(ops, "fused_moe_awq", fake_fused)
+    x, lg = torch.zeros((3, 256), dtype=torch.float16), torch.zeros((3, 4))
+    y = method.apply(moe_layer, x, lg, 2, True, use_grouped_topk=False, topk_group=None, num_expert_group=None,
+                     global_num_experts=4, expert_map=None, custom_routing_function=None, scoring_func="softmax",
+                     e_score_correction_bias=None, apply_router_weight_on_input=False, activation="silu")
+    assert tuple(y.shape) == (3, 256)
+    assert seen["topk"] == 2 and seen["renorm"] is True
+    assert tuple(seen["w13"]) == (4, 256, 32) and tuple(seen["w2"]) == (4, 128, 32)
+    with pytest.raises(NotImplementedError):
+        method.apply(moe_layer, x, lg, 2, True, apply_router_weight_on_input=True)
+
+
+def test_awq_gemm_takes_vllm_split_k_iters_as_a_hint(sba, monkeypatch):
+    """vLLM's AWQLinearMethod.apply always passes its pack factor (8) as split_k_iters.  The op
+    this package binds in its place must hand 0 (= the library's own choice) to the C ABI for
+    it, and only force_split_k reaches the library."""
+    import importlib
+    ops = importlib.import_module(sba.__name__ + ".ops")
+    libmod = importlib.import_module(sba.__name__ + "._lib")
+    calls = []
+
+    class FakeLib:
+        def awqmi_gemm_workspace_bytes(self, M, K, N, split):
+            calls.append(("ws", split))
+            return 65536
+
+        def awqmi_gemm_f16(self, *a):
+            calls.append(("gemm", a[11]))
+            return 0
+
+    monkeypatch.setattr(libmod, "load", lambda: FakeLib())
+    monkeypatch.setattr(ops, "_need", lambda *a, **k: None)
+    monkeypatch.setattr(ops, "_stream_ptr", lambda dev: 0)
+    monkeypatch.setattr(ops, "get_workspace", lambda dev, n, s=None: torch.zeros(n, dtype=torch.uint8))
+    monkeypatch.setattr(ops, "_gemm_ws_bytes", {})
+    x = torch.zeros((4, 256), dtype=torch.float16)
+    qw = torch.zeros((256, 16), dtype=torch.int32)
+    sc = torch.zeros((2, 128), dtype=torch.float16)
+    qz = torch.zeros((2, 16), dtype=torch.int32)
+    ops.awq_gemm(x, qw, sc, qz, 8)                       # what vLLM passes
+    assert calls == [("ws", 0), ("gemm", 0)]
+    calls.clear()
+    ops.awq_gemm(x, qw, sc, qz, 8, force_split_k=2)
+    assert calls == [("ws", 2), ("gemm", 2)]
+
+
+def test_plugin_entry_point_resolves_from_the_mounted_layout(sba):
+    """What deploy.py mounts into a server is the root of this repository on PYTHONPATH: the
+    .dist-info directory there must declare the vllm.general_plugins entry point, and the entry
+    point must load (through the `server_benchmark_amd` alias module beside it)."""
+    import importlib.metadata as md
+    dists = [d for d in md.distributions(path=[ROOT]) if d.metadata["Name"] == "server_benchmark_amd"]
+    assert len(dists) == 1
+    eps = [e for e in dists[0].entry_points if e.group == "vllm.general_plugins"]
+    assert [e.name for e in eps] == ["awq_mi355x"]
+    deploy = __import__("importlib").import_module(sba.__name__ + ".deploy")
+    assert eps[0].name == deploy.PLUGIN_NAME
+    fn = eps[0].load()
+    plugin = __import__("importlib").import_module(sba.__name__ + ".vllm_plugin")
+    assert fn is plugin.register
+    assert os.path.exists(os.path.join(ROOT, "server_benchmark_amd.py"))      # the alias the entry point names
