@@ -114,6 +114,10 @@ def main():
     lib = _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    st = lib.awqmi_init()        # the library's one-time set-up, as a binding does after loading it
+    if st != 0:
+        log(f"bench.py: awqmi_init failed: {lib.awqmi_status_string(st).decode()}")
+        sys.exit(1)
     gen = torch.Generator(device=dev).manual_seed(0)
     G = 128
     layers = workloads.QWEN25_72B_LAYERS
