@@ -49,10 +49,11 @@ typedef enum awqmi_status {
 /* Optional one-time set-up on the current device: raises the dynamic-LDS limit of the kernels
  * that need it, looks up this GPU's static scratch array (awqmi_gemm_f16_noalloc) and zeroes its
  * arrival counters (synchronously, on the null stream).  Every entry point does its share of
- * this on its first use; call this once after loading the library if the first use may sit
- * inside a stream capture.  The library assumes
- * one GPU per process (the harness starts one server process per replica and GPU set,
- * reference utils/generate_compose.py:85-100). */
+ * this on its first use; call this once per device after loading the library if the first use
+ * on that device may sit inside a stream capture.  All set-up state is kept per device (the
+ * harness starts one server process per replica and GPU set, reference
+ * utils/generate_compose.py:85-100; a process that drives several GPUs makes each one current
+ * for its own calls). */
 int awqmi_init(void);
 int awqmi_version(void);
 const char* awqmi_status_string(int status);

@@ -228,10 +228,13 @@ int mfma_pick_rows(int M, int K, int N) {
 }  // namespace
 
 // Kernels that use more dynamic LDS than the default limit need a function attribute; it is
-// set once per process for all of them (by awqmi_init, or by the first call that needs one).
+// set once per device for all of them (by awqmi_init, or by the first call on that device that
+// needs one).
 static int ensure_kernel_attributes() {
-  static std::atomic<bool> done{false};
-  if (done.load(std::memory_order_acquire)) return AWQMI_OK;
+  static std::atomic<bool> done[MAX_DEVICES];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) dev = 0;
+  if (done[dev].load(std::memory_order_acquire)) return AWQMI_OK;
   const void* mfma[] = {
       reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1, 8>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1, 8>),
       reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 2, 8>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 2, 8>),
@@ -257,7 +260,7 @@ static int ensure_kernel_attributes() {
                                              (MOE_ALIGN_WAVES + 2) * AWQMI_MAX_EXPERTS * (int)sizeof(int));
     if (e != hipSuccess) { t_last_hip_error = (int)e; return AWQMI_LAUNCH_FAILED; }
   }
-  done.store(true, std::memory_order_release);
+  done[dev].store(true, std::memory_order_release);
   return AWQMI_OK;
 }
 
