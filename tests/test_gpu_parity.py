@@ -242,6 +242,33 @@ def test_gemm_workspace_counters_stay_zero(sba, gpu):
     assert int(ws[:65536].view(torch.int32).abs().sum().item()) == 0
 
 
+def test_split_k_exchange_is_stable_over_many_launches_and_two_streams(sba, gpu):
+    """The split-K hand-off (partial tiles + arrival counters in the workspace) over a few thousand
+    launches: shapes alternate on one stream and share its workspace, a second stream with a
+    workspace of its own runs the same calls at the same time, and every result must carry the bits
+    of the first one."""
+    cases = []
+    for M, K, N, seed in ((16, 4096, 2048, 1), (1, 8192, 1024, 2), (7, 2048, 264, 3), (32, 4096, 512, 4)):
+        x, qw, s, qz = _np_case(M, K, N, 128, seed=seed)
+        cases.append(_dev(gpu, x, qw, s, qz))
+    first = [sba.awq_gemm(*c, 0).clone() for c in cases]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    outs = {0: [], 1: []}
+    for it in range(400):
+        for i, c in enumerate(cases):
+            outs[0].append((i, sba.awq_gemm(*c, 0)))
+            with torch.cuda.stream(side):
+                outs[1].append((i, sba.awq_gemm(*c, 0)))
+        if it % 50 == 49:               # compare in batches, so that launches queue up back to back
+            torch.cuda.synchronize()
+            for k in (0, 1):
+                for i, y in outs[k]:
+                    assert torch.equal(y, first[i]), (it, k, i)
+                outs[k].clear()
+    torch.cuda.synchronize()
+
+
 def test_workspace_reset_zeroes_the_counters(sba, gpu):
     """A workspace whose counters were left non-zero (a call cut short) gives wrong split-K sums
     until it is reset; awqmi_workspace_reset puts it back."""
