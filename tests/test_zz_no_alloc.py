@@ -96,3 +96,39 @@ def test_noalloc_gemm_refuses_what_does_not_fit(gpu):
                                       M, K, N, G, 0, st) == 6
     assert lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), y.data_ptr(),
                                       M, K, N + 4, G, 0, st) == 1
+
+
+def test_noalloc_gemm_replays_from_a_captured_graph(gpu):
+    """What the entry point is for: a call recorded into a HIP graph with no workspace to carry.
+    Replays, with other calls of the entry point and eager work in between, must reproduce the
+    eager result bit for bit."""
+    from server_benchmark_amd import _lib
+    lib = _lib.load()
+    assert lib.awqmi_init() == 0                      # set-up outside the capture
+    M, K, N, G = 8, 4096, 2048, 128
+    x, qw, sc, qz = _case(M, K, N, G, gpu, 11)
+    y_eager = torch.empty((M, N), dtype=torch.float16, device=gpu)
+    y_graph = torch.zeros((M, N), dtype=torch.float16, device=gpu)
+
+    def call(y, stream):
+        rc = lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), y.data_ptr(),
+                                        M, K, N, G, 0, stream)
+        assert rc == 0, lib.awqmi_status_string(rc).decode()
+
+    assert lib.awqmi_gemm_auto_split_k(M, K, N, G) > 1            # the scratch array is really in use
+    call(y_eager, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            call(y_graph, s.cuda_stream)
+        for _ in range(3):
+            y_graph.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y_graph.view(torch.int16), y_eager.view(torch.int16))
+            other, _ = _both(lib, gpu, 3, 1024, 512, 128, 4, 12)       # eager calls on the same array in between
+            assert torch.isfinite(other).all()
+    torch.cuda.current_stream().wait_stream(s)
