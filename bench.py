@@ -373,66 +373,84 @@ def main():
     if not args.no_prefill:
         mq = workloads.QWEN3_MOE
         H, E, topk, I = mq["hidden"], mq["experts"], mq["topk"], mq["inter"]
-        w13 = [make_weights(H, 2 * I, G, dev, gen) for _ in range(E)]
-        w2 = [make_weights(I, H, G, dev, gen) for _ in range(E)]
-        w13 = tuple(torch.stack([w[i] for w in w13]) for i in range(3))
-        w2 = tuple(torch.stack([w[i] for w in w2]) for i in range(3))
+        # Sixteen weight sets (the experts of sixteen layers, 5 GB), one per call of a 16-call graph:
+        # between two uses of a set the other fifteen stream through, so even at T = 1 (8 experts,
+        # 20 MB per call) the weights come from HBM and not from the 256 MB Infinity Cache, as they
+        # do in a decoder whose every layer has experts of its own.  The cache-warm figure (one set,
+        # every call on the same experts) is reported beside it.
+        NSETS = 16
+
+        def expert_set():
+            lo, hi = -(2 ** 31), 2 ** 31
+            def triple(K, N):
+                return (torch.randint(lo, hi, (E, K, N // 8), dtype=torch.int32, device=dev, generator=gen),
+                        (torch.rand((E, K // G, N), device=dev, generator=gen) * 0.019 + 0.001).to(torch.float16),
+                        torch.randint(lo, hi, (E, K // G, N // 8), dtype=torch.int32, device=dev, generator=gen))
+            return triple(H, 2 * I), triple(I, H)
+
+        sets = [expert_set() for _ in range(NSETS)]
         mo = []
+
+        def graph_us(calls, n_it=20):
+            """calls: list of (x, w13, w2, logits); one graph holding them all, replayed; us per call."""
+            gs = torch.cuda.Stream()
+            gs.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(gs):
+                ys = [sba.fused_moe_awq(x_, a_, b_, l_, topk, True).clone() for x_, a_, b_, l_ in calls]   # sizes the workspace
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=gs):
+                    yg = [sba.fused_moe_awq(x_, a_, b_, l_, topk, True) for x_, a_, b_, l_ in calls]
+                for _ in range(3):
+                    graph.replay()
+                torch.cuda.synchronize()
+                ea, eb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                ea.record()
+                for _ in range(n_it):
+                    graph.replay()
+                eb.record()
+                torch.cuda.synchronize()
+            torch.cuda.current_stream().wait_stream(gs)
+            for i, (y1, y2) in enumerate(zip(ys, yg)):
+                if not torch.equal(y1, y2):
+                    raise RuntimeError(f"MoE block: call {i} of the replayed graph differs from the eager call")
+            return ea.elapsed_time(eb) * 1e3 / (n_it * len(calls))
+
         for T in workloads.MOE_T:
             xm = torch.randn((T, H), device=dev, generator=gen).to(torch.float16)
-            lg = torch.randn((T, E), device=dev, generator=gen)
+            lgs = [torch.randn((T, E), device=dev, generator=gen) for _ in range(NSETS)]
+            distinct = sum(int(torch.unique(sba.topk_softmax(l_, topk, True)[1]).numel()) for l_ in lgs) / NSETS
+            w13_0, w2_0 = sets[0]
             for _ in range(3):
-                ym = sba.fused_moe_awq(xm, w13, w2, lg, topk, True)
+                sba.fused_moe_awq(xm, w13_0, w2_0, lgs[0], topk, True)
             torch.cuda.synchronize()
-            _, ids = sba.topk_softmax(lg, topk, True)
-            distinct = int(torch.unique(ids).numel())
             n_it = 20
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a.record()
             for _ in range(n_it):
-                ym = sba.fused_moe_awq(xm, w13, w2, lg, topk, True)
+                sba.fused_moe_awq(xm, w13_0, w2_0, lgs[0], topk, True)
             b.record()
             torch.cuda.synchronize()
             us_eager = a.elapsed_time(b) * 1e3 / n_it
-            # the same call replayed from a HIP graph (how a serving engine runs decode steps)
-            gs = torch.cuda.Stream()
-            gs.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(gs):
-                ym = sba.fused_moe_awq(xm, w13, w2, lg, topk, True)      # sizes this stream's workspace
-                torch.cuda.synchronize()
-                graph = torch.cuda.CUDAGraph()
-                # eight calls per graph: a serving engine's graph holds a whole decode step (many
-                # layers), so the launch gap between two replays is not part of a block's time
-                per_graph = 8
-                with torch.cuda.graph(graph, stream=gs):
-                    for _ in range(per_graph):
-                        yg = sba.fused_moe_awq(xm, w13, w2, lg, topk, True)
-                for _ in range(3):
-                    graph.replay()
-                torch.cuda.synchronize()
-                a.record()
-                for _ in range(n_it):
-                    graph.replay()
-                b.record()
-                torch.cuda.synchronize()
-            torch.cuda.current_stream().wait_stream(gs)
-            us = a.elapsed_time(b) * 1e3 / (n_it * per_graph)
-            if not torch.equal(yg, ym):
-                raise RuntimeError(f"MoE block T={T}: graph replay differs from the eager call")
-            del graph
-            nbytes = workloads.moe_bytes(distinct, T, H, I, G)
+            # replayed from a HIP graph (how a serving engine runs decode steps; a graph holds many
+            # layers, so the launch gap between two replays is not part of a block's time)
+            us = graph_us([(xm, sets[i][0], sets[i][1], lgs[i]) for i in range(NSETS)])
+            us_warm = graph_us([(xm, w13_0, w2_0, lgs[0])] * 8)
+            nbytes = workloads.moe_bytes(1, T, H, I, G) * 0 + distinct * workloads.moe_bytes(1, 0, H, I, G) + 2 * (T * H * 2)
             fl = workloads.moe_flops(T, topk, H, I)
-            mo.append({"T": T, "distinct_experts": distinct, "us": round(us, 1), "us_eager_call": round(us_eager, 1),
+            mo.append({"T": T, "distinct_experts": round(distinct, 1), "us": round(us, 1),
+                       "us_cache_warm": round(us_warm, 1), "us_eager_call": round(us_eager, 1),
                        "GBps": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                        "TFLOPs": round(fl / us / 1e6, 2), "frac_mfma": round(fl / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 5)})
             if args.detail:
-                log(f"   moe T={T:4d} experts hit {distinct:3d}  {us:9.1f} us (eager call {us_eager:6.1f})  "
-                    f"{nbytes / us / 1e3:8.1f} GB/s")
+                log(f"   moe T={T:4d} experts hit {distinct:5.1f}  {us:9.1f} us from HBM ({us_warm:6.1f} cache-warm, eager "
+                    f"call {us_eager:6.1f})  {nbytes / us / 1e3:8.1f} GB/s")
         out["moe"] = {"workload": "Qwen3-30B-A3B MoE block: route + align + grouped w13 GEMM + SiLU*up + grouped w2 "
-                                  "GEMM + slot sum, 128 experts, top-8, hidden 2048, inter 768 (whole block per call, "
-                                  "eight calls per HIP graph, graph replayed; weights not rotated: cache-warm for small T)",
+                                  "GEMM + slot sum, 128 experts, top-8, hidden 2048, inter 768; whole block per call, "
+                                  "16 calls per HIP graph on 16 different expert sets and routings (weights from HBM), "
+                                  "graph replayed; us_cache_warm: 8 calls per graph on one set",
                       "points": mo}
-        del w13, w2
+        del sets
 
     # ------------------------------------------------------------------ serving-shaped decoder load (opt-in)
     if not args.no_decoder and not args.sweep_only and args.pmc_target is None:
