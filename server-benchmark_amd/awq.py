@@ -3,10 +3,13 @@ drives for an AWQ checkpoint (the servers the benchmark harness starts at refere
 utils/generate_compose.py:85-93 pick this method from the checkpoint's quantization_config
 because no --quantization flag is passed).  Same method names, argument meaning and registered
 parameter names (`qweight`, `qzeros`, `scales`), so AWQ state dicts load unchanged; the
-layers are plain torch.nn.Module objects and nothing here imports vLLM.
+layers are plain torch.nn.Module objects.  vLLM is never required: the only place that looks
+for it is create_weights, which wraps the parameters in vLLM's own parameter classes when those
+can be imported, because vLLM's shard-aware weight loaders call methods of these classes.
 """
 from __future__ import annotations
 
+import importlib
 from typing import Any, Optional
 
 import torch
@@ -93,6 +96,21 @@ def _register(layer, name, tensor, attrs: dict[str, Any]):
     layer.register_parameter(name, p)
 
 
+def _vllm_parameter_classes():
+    """(PackedvLLMParameter, GroupQuantScaleParameter) of vllm.model_executor.parameter, or None
+    outside vLLM.  vLLM's linear layers pick their second-generation weight loader by the class
+    NAME of the quantisation method, and `AWQLinearMethod` is on that list; that loader calls
+    shard-loading methods (load_column_parallel_weight, load_merged_column_weight,
+    load_qkv_weight, load_row_parallel_weight) that only these parameter classes have."""
+    try:
+        mod = importlib.import_module("vllm.model_executor.parameter")
+    except ImportError:
+        return None
+    packed = getattr(mod, "PackedvLLMParameter", None)
+    scale = getattr(mod, "GroupQuantScaleParameter", None)
+    return (packed, scale) if packed is not None and scale is not None else None
+
+
 class AWQLinearMethod:
     def __init__(self, quant_config: AWQConfig):
         self.quant_config = quant_config
@@ -113,16 +131,27 @@ class AWQLinearMethod:
             raise ValueError("AWQ scales / activations must be float16")
         dev = extra_weight_attrs.pop("device", None)
         ngroups = input_size_per_partition // group
-        packed = dict(input_dim=0, output_dim=1, packed_dim=1, pack_factor=cfg.pack_factor)
-        _register(layer, "qweight",
-                  torch.empty(input_size_per_partition, out_pp // cfg.pack_factor, dtype=torch.int32, device=dev),
-                  {**packed, **extra_weight_attrs})
-        _register(layer, "qzeros",
-                  torch.empty(ngroups, out_pp // cfg.pack_factor, dtype=torch.int32, device=dev),
-                  {**packed, **extra_weight_attrs})
-        _register(layer, "scales",
-                  torch.empty(ngroups, out_pp, dtype=params_dtype, device=dev),
-                  {"input_dim": 0, "output_dim": 1, **extra_weight_attrs})
+        qweight = torch.empty(input_size_per_partition, out_pp // cfg.pack_factor, dtype=torch.int32, device=dev)
+        qzeros = torch.empty(ngroups, out_pp // cfg.pack_factor, dtype=torch.int32, device=dev)
+        scales = torch.empty(ngroups, out_pp, dtype=params_dtype, device=dev)
+        weight_loader = extra_weight_attrs.get("weight_loader")
+        classes = _vllm_parameter_classes() if callable(weight_loader) else None
+        if classes is not None:
+            # inside vLLM: its parameter classes, built the way its own AWQ method builds them
+            packed_cls, scale_cls = classes
+            layer.register_parameter("qweight", packed_cls(
+                data=qweight, input_dim=0, output_dim=1, packed_dim=1, packed_factor=cfg.pack_factor,
+                weight_loader=weight_loader))
+            layer.register_parameter("qzeros", packed_cls(
+                data=qzeros, input_dim=0, output_dim=1, packed_dim=1, packed_factor=cfg.pack_factor,
+                weight_loader=weight_loader))
+            layer.register_parameter("scales", scale_cls(
+                data=scales, input_dim=0, output_dim=1, weight_loader=weight_loader))
+        else:
+            packed = dict(input_dim=0, output_dim=1, packed_dim=1, pack_factor=cfg.pack_factor)
+            _register(layer, "qweight", qweight, {**packed, **extra_weight_attrs})
+            _register(layer, "qzeros", qzeros, {**packed, **extra_weight_attrs})
+            _register(layer, "scales", scales, {"input_dim": 0, "output_dim": 1, **extra_weight_attrs})
         layer.input_size_per_partition = input_size_per_partition
         layer.output_size_per_partition = out_pp
         layer.output_partition_sizes = list(output_partition_sizes)
@@ -176,8 +205,13 @@ class AWQMoEMethod:
             "w2_scales": ((num_experts, grp(I), hidden_size), params_dtype),
             "w2_qzeros": ((num_experts, grp(I), hidden_size // pf), torch.int32),
         }
+        # Attributes vLLM's FusedMoE.weight_loader reads off a parameter: AWQ stores a weight as
+        # [K, N / 8] (input dimension first), which that loader calls "transposed" and needs to
+        # know to shard gate / up along the last dimension; "group" is its name for scales and
+        # zero points that come one per quantisation group.
+        attrs = {"is_transposed": True, "quant_method": "group", **extra_weight_attrs}
         for name, (shape, dt) in shapes.items():
-            _register(layer, name, torch.empty(shape, dtype=dt, device=dev), dict(extra_weight_attrs))
+            _register(layer, name, torch.empty(shape, dtype=dt, device=dev), dict(attrs))
 
     def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
         for name in ("w13_qweight", "w13_scales", "w13_qzeros", "w2_qweight", "w2_scales", "w2_qzeros"):

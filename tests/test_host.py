@@ -338,6 +338,27 @@ def _fake_vllm(monkeypatch, with_registry=True):
         mod("vllm.model_executor.layers.quantization.base_config", QuantizationConfig=QuantizationConfig)
         mod("vllm.model_executor.layers.fused_moe", FusedMoE=FusedMoE)
         mod("vllm.model_executor.layers.linear", LinearBase=LinearBase)
+
+        class _ShardAware(torch.nn.Parameter):       # vLLM's parameter classes: keyword-only, loader-carrying
+            def __new__(cls, data, **kw):
+                return super().__new__(cls, data=data, requires_grad=False)
+
+            def __init__(self, data, weight_loader, input_dim, output_dim, **kw):
+                self.built_with = dict(weight_loader=weight_loader, input_dim=input_dim, output_dim=output_dim, **kw)
+
+            def load_merged_column_weight(self, *a, **k):
+                return "sharded"
+
+        class PackedvLLMParameter(_ShardAware):
+            def __init__(self, data, weight_loader, input_dim, output_dim, packed_dim, packed_factor, **kw):
+                super().__init__(data, weight_loader, input_dim, output_dim, packed_dim=packed_dim,
+                                 packed_factor=packed_factor, **kw)
+
+        class GroupQuantScaleParameter(_ShardAware):
+            pass
+
+        mod("vllm.model_executor.parameter", PackedvLLMParameter=PackedvLLMParameter,
+            GroupQuantScaleParameter=GroupQuantScaleParameter)
     return mods
 
 
@@ -407,6 +428,46 @@ def test_vllm_plugin_registers_the_awq_method_for_linear_and_moe_layers(sba, mon
     assert tuple(seen["w13"]) == (4, 256, 32) and tuple(seen["w2"]) == (4, 128, 32)
     with pytest.raises(NotImplementedError):
         method.apply(moe_layer, x, lg, 2, True, apply_router_weight_on_input=True)
+
+
+def test_create_weights_uses_vllm_parameter_classes_inside_vllm(sba, monkeypatch):
+    """vLLM picks its second-generation weight loader for a method whose class is NAMED
+    AWQLinearMethod, and that loader calls shard-loading methods of vLLM's parameter classes: with
+    vLLM importable and a callable weight_loader the three parameters are built from those classes
+    (same keyword arguments as vLLM's own AWQ method), keep their names, shapes and dtypes, and
+    turn into plain contiguous parameters after loading."""
+    mods = _fake_vllm(monkeypatch)
+    par = mods["vllm.model_executor.parameter"]
+    loader = lambda param, loaded, *a: None
+    assert sba.AWQLinearMethod.__name__ == "AWQLinearMethod"
+    m = sba.AWQLinearMethod(sba.AWQConfig(4, 128, True))
+    layer = torch.nn.Module()
+    m.create_weights(layer, 1024, [512, 128, 128], 1024, 768, torch.float16, weight_loader=loader)
+    assert type(layer.qweight) is par.PackedvLLMParameter and type(layer.qzeros) is par.PackedvLLMParameter
+    assert type(layer.scales) is par.GroupQuantScaleParameter
+    assert layer.qweight.built_with == dict(weight_loader=loader, input_dim=0, output_dim=1, packed_dim=1,
+                                            packed_factor=8)
+    assert layer.scales.built_with == dict(weight_loader=loader, input_dim=0, output_dim=1)
+    assert layer.qweight.load_merged_column_weight() == "sharded"
+    assert tuple(layer.qweight.shape) == (1024, 96) and layer.qweight.dtype == torch.int32
+    assert tuple(layer.qzeros.shape) == (8, 96) and tuple(layer.scales.shape) == (8, 768)
+    assert sorted(n for n, _ in layer.named_parameters()) == ["qweight", "qzeros", "scales"]
+    m.process_weights_after_loading(layer)
+    assert type(layer.qweight) is torch.nn.Parameter and layer.qweight.is_contiguous()
+    # no loader given (this package's own checkpoint reader): plain parameters with the attributes
+    l2 = torch.nn.Module()
+    m.create_weights(l2, 1024, [768], 1024, 768, torch.float16)
+    assert type(l2.qweight) is torch.nn.Parameter and l2.qweight.pack_factor == 8
+
+
+def test_moe_parameters_carry_what_vllms_expert_loader_reads(sba):
+    m = sba.AWQMoEMethod(sba.AWQConfig(4, 128, True))
+    layer = torch.nn.Module()
+    loader = lambda *a, **k: None
+    m.create_weights(layer, 4, 256, 128, torch.float16, weight_loader=loader)
+    for name in ("w13_qweight", "w13_scales", "w13_qzeros", "w2_qweight", "w2_scales", "w2_qzeros"):
+        p = getattr(layer, name)
+        assert p.is_transposed is True and p.quant_method == "group" and p.weight_loader is loader
 
 
 def test_awq_gemm_takes_vllm_split_k_iters_as_a_hint(sba, monkeypatch):
