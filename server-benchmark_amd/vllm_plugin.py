@@ -45,13 +45,15 @@ def _optional(module: str, attr: str):
 def make_vllm_config_class():
     """This package's AWQConfig as a subclass of vLLM's QuantizationConfig (when that base class
     can be imported), choosing the layer method by vLLM's own layer classes: FusedMoE layers get
-    AWQMoEMethod, linear layers AWQLinearMethod, everything else (and every module listed in
-    modules_to_not_convert) stays unquantised."""
+    AWQMoEMethod, linear layers AWQLinearMethod, everything else stays unquantised (None).  A
+    linear layer listed in modules_to_not_convert gets vLLM's UnquantizedLinearMethod, as vLLM's
+    own AWQ config answers: vLLM's linear layers call the returned method unconditionally."""
     from .awq import AWQConfig, AWQLinearMethod, AWQMoEMethod
 
     base = _optional(_QUANT_PKG + ".base_config", "QuantizationConfig")
     fused_moe_cls = _optional("vllm.model_executor.layers.fused_moe", "FusedMoE")
     linear_cls = _optional("vllm.model_executor.layers.linear", "LinearBase")
+    unquantized_linear = _optional("vllm.model_executor.layers.linear", "UnquantizedLinearMethod")
     bases = (AWQConfig,) if base is None else (AWQConfig, base)
 
     class MI355XAWQConfig(*bases):
@@ -68,6 +70,8 @@ def make_vllm_config_class():
 
         def get_quant_method(self, layer, prefix=""):
             if self.is_skipped(prefix):
+                if linear_cls is not None and unquantized_linear is not None and isinstance(layer, linear_cls):
+                    return unquantized_linear()
                 return None
             if (fused_moe_cls is not None and isinstance(layer, fused_moe_cls)) or getattr(layer, "is_fused_moe", False):
                 return AWQMoEMethod(self)

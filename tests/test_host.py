@@ -331,13 +331,16 @@ def _fake_vllm(monkeypatch, with_registry=True):
         class LinearBase(torch.nn.Module):
             pass
 
+        class UnquantizedLinearMethod:
+            pass
+
         mod("vllm.model_executor")
         mod("vllm.model_executor.layers")
         mod("vllm.model_executor.layers.quantization", QUANTIZATION_METHODS=["awq", "gptq", "awq_marlin"],
             _CUSTOMIZED_METHOD_TO_QUANT_CONFIG={})
         mod("vllm.model_executor.layers.quantization.base_config", QuantizationConfig=QuantizationConfig)
         mod("vllm.model_executor.layers.fused_moe", FusedMoE=FusedMoE)
-        mod("vllm.model_executor.layers.linear", LinearBase=LinearBase)
+        mod("vllm.model_executor.layers.linear", LinearBase=LinearBase, UnquantizedLinearMethod=UnquantizedLinearMethod)
 
         class _ShardAware(torch.nn.Parameter):       # vLLM's parameter classes: keyword-only, loader-carrying
             def __new__(cls, data, **kw):
@@ -407,7 +410,11 @@ def test_vllm_plugin_registers_the_awq_method_for_linear_and_moe_layers(sba, mon
     moe_layer = mods["vllm.model_executor.layers.fused_moe"].FusedMoE()
     lin_layer = mods["vllm.model_executor.layers.linear"].LinearBase()
     assert isinstance(cfg.get_quant_method(lin_layer, "model.layers.0.self_attn.qkv_proj"), sba.AWQLinearMethod)
-    assert cfg.get_quant_method(lin_layer, "model.layers.0.mlp.gate.") is None        # the router stays fp16
+    # the router stays fp16: a skipped linear layer gets vLLM's unquantised method (vLLM's linear
+    # layers call whatever is returned), any other skipped module None
+    skipped = cfg.get_quant_method(lin_layer, "model.layers.0.mlp.gate.")
+    assert isinstance(skipped, mods["vllm.model_executor.layers.linear"].UnquantizedLinearMethod)
+    assert cfg.get_quant_method(torch.nn.LayerNorm(4), "model.layers.0.mlp.gate.norm") is None
     assert cfg.get_quant_method(torch.nn.LayerNorm(4), "model.norm") is None
     method = cfg.get_quant_method(moe_layer, "model.layers.0.mlp.experts")
     assert isinstance(method, sba.AWQMoEMethod)
