@@ -24,6 +24,8 @@
  *   1 << 19  awq_gemm with 17..64 rows: the MFMA kernel wherever it can run
  *   1 << 20  v = bits 20..22: MFMA tiles of 64 v rows (v = 1..4) whatever M is
  *   1 << 23  dense skinny launches never share left-over chunks step by step
+ *   1 << 24  the one-call MoE block always routes in a launch of its own (blocks of at most four
+ *            tokens otherwise fold the routing into the first expert GEMM)
  * The workspace must be large enough for the form that is forced: the sizes the public queries
  * return cover every variant except a forced MFMA tile size, which silently runs without its K
  * split when the workspace is too small for it.

@@ -57,6 +57,7 @@ enum : int {
   VAR_MID_M_MFMA = 1 << 19,   // awq_gemm with 17..64 rows: the MFMA kernel wherever it can run
   VAR_MFMA_ROWS_SHIFT = 20,   // bits 20..22 = v: MFMA tiles of 64 v rows (v = 1..4) whatever M is
   VAR_NO_TAIL_STEP = 1 << 23, // dense skinny launches never share left-over chunks step by step
+  VAR_NO_FOLDED_ROUTE = 1 << 24, // the one-call MoE block always routes in a launch of its own
 };
 inline bool variant_on(int bit) {
   return t_variant >= 0 && (t_variant & bit);
@@ -286,6 +287,40 @@ static int moe_route_align_small(const float* logits, int T, int E, int topk, in
   if (E <= 256) return moe_route_align_launch<4>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
   if (E <= 512) return moe_route_align_launch<8>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
   return moe_route_align_launch<16>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
+}
+
+// Routing of one MoE block: inputs and the five lists it produces.
+struct MoeRoute {
+  const float* logits;
+  const float* bias;
+  int T, E, topk, scoring, renorm;
+  float scale;
+  int32_t* ids;
+  float* wts;
+  int32_t* sorted;
+  int32_t* experts;
+  int32_t* npp;
+};
+
+// Routing + align of a short slot list as launches of their own (one launch for plain softmax
+// routing of up to 16 tokens, else top-k and align apart).
+static int moe_route_launches(const MoeRoute& r, int tile, void* stream) {
+  const bool plain = r.scoring == 0 && !r.bias && r.scale == 1.f;
+  if (r.T <= MOE_ALIGN_WAVES && plain)
+    return moe_route_align_small(r.logits, r.T, r.E, r.topk, r.renorm, r.ids, r.wts, tile, r.sorted, r.experts, r.npp,
+                                 stream);
+  if (const int st = awqmi_moe_topk_f32(r.logits, r.bias, r.T, r.E, r.topk, r.scoring, r.renorm, r.scale, r.ids, r.wts,
+                                        stream))
+    return st;
+  return awqmi_moe_align(r.ids, r.T * r.topk, r.E, tile, r.sorted, r.experts, r.npp, stream);
+}
+
+// Folded routing: at most four tokens (one per wave of a workgroup; the kernel would take up to
+// eight in turn, but from five tokens on every workgroup spends on the second round what the
+// saved launch gains: 128 experts, top-8, weights from HBM: 3.5 us of 29 - 38 faster at 1 - 4
+// tokens, 0.9 us at 5, nothing at 6 - 8), 64 slots (one lane each), 128 experts (two per lane).
+static bool moe_route_foldable(int T, int E, int topk, int tile) {
+  return T <= 4 && T * topk <= 64 && E <= 128 && tile == 16 && !variant_on(VAR_NO_FOLDED_ROUTE);
 }
 
 extern "C" {
@@ -578,7 +613,11 @@ int awqmi_moe_align(const int32_t* topk_ids, int n_slots, int E, int tile_m, int
 
 // sorted-token blocks a grouped launch covers: the align capacity, rounded up to whole groups
 static int moe_launch_blocks(int n_slots, int E, int tile_m) {
-  const int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, tile_m) / tile_m);
+  int nblk = (int)(awqmi_moe_align_capacity(n_slots, E, tile_m) / tile_m);
+  // a block that runs holds at least one real slot: a handful of tokens never fills more blocks
+  // than it has slots, whatever the expert count (one token with 8 picks of 128 experts: 8
+  // blocks, not 121 -- the rest would be workgroups that start, read the padded count and leave)
+  if (nblk > n_slots) nblk = n_slots;
   return (nblk + MOE_BLOCK_GROUP_MAX - 1) / MOE_BLOCK_GROUP_MAX * MOE_BLOCK_GROUP_MAX;
 }
 
@@ -643,7 +682,8 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
                          void* y, const int32_t* sorted_token_ids, const int32_t* expert_ids,
                          const int32_t* num_tokens_post_padded, const float* topk_weights, int n_slots,
                          int a_row_div, int tile_m, int E, int K, int N, int group, int split_k,
-                         void* workspace, size_t workspace_bytes, void* stream, bool fuse_act);
+                         void* workspace, size_t workspace_bytes, void* stream, bool fuse_act,
+                         const MoeRoute* route = nullptr);
 
 int awqmi_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
                        void* y, const int32_t* sorted_token_ids, const int32_t* expert_ids,
@@ -659,7 +699,10 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
                          void* y, const int32_t* sorted_token_ids, const int32_t* expert_ids,
                          const int32_t* num_tokens_post_padded, const float* topk_weights, int n_slots,
                          int a_row_div, int tile_m, int E, int K, int N, int group, int split_k,
-                         void* workspace, size_t workspace_bytes, void* stream, bool fuse_act) {
+                         void* workspace, size_t workspace_bytes, void* stream, bool fuse_act,
+                         const MoeRoute* route) {
+  // route: the block's routing has not run yet.  The launch takes it along when it is the plain
+  // 16-row-block form with G = 128; any other form routes in launches of its own first.
   if (!x || !qweight || !scales || !qzeros || !y || !sorted_token_ids || !expert_ids ||
       !num_tokens_post_padded)
     return AWQMI_NULL_POINTER;
@@ -677,6 +720,8 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   if (tile_m >= 64) {
     // blocks of 64 / 128 slots: the MFMA kernel in its expert-grouped form (no K split)
     if (fuse_act) return AWQMI_BAD_ARGUMENT;
+    if (route)
+      if (const int rc = moe_route_launches(*route, tile_m, stream)) return rc;
     const size_t x_rows = ((size_t)n_slots + a_row_div - 1) / a_row_div;
     if (x_rows * K * 2 >= (1ull << 32) || (size_t)K * NW * 4 >= (1ull << 32) ||
         (size_t)(K / G) * N * 2 >= (1ull << 32))
@@ -772,6 +817,24 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   // HBM rather than from a warm cache)
   const bool ldsq = wpl == 2 && tile_m == 16 && (size_t)K * NW * 4 < (1ull << 31) &&
                     (long long)n_slots >= 16LL * E && !variant_on(VAR_NO_LDS_RING);
+  const bool plain_form = !ldsq && !act_pair &&
+                          (act_split || (tile_m == 16 && wpl == 2 && !pair_cols && !variant_on(VAR_MOE_RING4)));
+  if (route) {
+    if (plain_form && G == 128 && moe_route_foldable(route->T, route->E, route->topk, tile_m)) {
+      p.r_logits = route->logits; p.r_bias = route->bias;
+      p.r_T = route->T; p.r_E = route->E; p.r_topk = route->topk; p.r_renorm = route->renorm;
+      p.r_scale = route->scale;
+      p.r_ids = route->ids; p.r_wts = route->wts; p.r_sorted = route->sorted; p.r_experts = route->experts;
+      p.r_npp = route->npp;
+      const bool two = route->E > 64, sig = route->scoring == 1;
+      if (two && sig) hipLaunchKernelGGL((awq_gemv_route_kernel<2, 2, true>), grid, dim3(256), 0, st, p);
+      else if (two) hipLaunchKernelGGL((awq_gemv_route_kernel<2, 2, false>), grid, dim3(256), 0, st, p);
+      else if (sig) hipLaunchKernelGGL((awq_gemv_route_kernel<2, 1, true>), grid, dim3(256), 0, st, p);
+      else hipLaunchKernelGGL((awq_gemv_route_kernel<2, 1, false>), grid, dim3(256), 0, st, p);
+      return launch_status();
+    }
+    if (const int rc = moe_route_launches(*route, tile_m, stream)) return rc;
+  }
   if (ldsq && act_pair) launch_gemv<2, 1, true, 4, 2, true, true>(p, grid, st);
   else if (ldsq && pair_cols && !act_split) launch_gemv<2, 1, true, 4, 2, false, true>(p, grid, st);
   else if (ldsq) launch_gemv<2, 1, true, 4, 4, false, true>(p, grid, st);
@@ -939,33 +1002,35 @@ int awqmi_fused_moe_routed_f16(const void* hidden, const float* router_logits, c
   void* act = ws + L.act;
   void* o = ws + L.o;
   int st;
-  const bool plain_routing = scoring == 0 && !score_bias && routed_scale == 1.f;
-  if (T <= MOE_ALIGN_WAVES && plain_routing) {
-    st = moe_route_align_small(router_logits, T, E, topk, renormalize, ids, wts, tile, sorted, experts, npp, stream);
+  const MoeRoute route{router_logits, score_bias, T, E, topk, scoring, renormalize, routed_scale,
+                       ids, wts, sorted, experts, npp};
+  // a handful of tokens: the first expert GEMM takes the routing along (one launch less)
+  const bool fold = moe_route_foldable(T, E, topk, tile);
+  const MoeRoute* pending = fold ? &route : nullptr;
+  if (fold) {
+    // nothing to launch here
+  } else if (L.n_slots < MOE_ALIGN_SPLIT_MIN || variant_on(VAR_ALIGN_ONE_WG)) {
+    st = moe_route_launches(route, tile, stream);
     if (st) return st;
   } else {
     st = awqmi_moe_topk_f32(router_logits, score_bias, T, E, topk, scoring, renormalize, routed_scale, ids, wts,
                             stream);
     if (st) return st;
-    if (L.n_slots >= MOE_ALIGN_SPLIT_MIN && !variant_on(VAR_ALIGN_ONE_WG)) {
-      // long slot lists: count per part, scan, place per part (three launches, many workgroups)
-      if (const int rc = ensure_kernel_attributes()) return rc;
-      int parts = (L.n_slots + 4095) / 4096;
-      if (parts > MOE_ALIGN_PARTS_MAX) parts = MOE_ALIGN_PARTS_MAX;
-      const int part = ((L.n_slots + parts - 1) / parts + 63) / 64 * 64;
-      parts = (L.n_slots + part - 1) / part;
-      int32_t* tab = reinterpret_cast<int32_t*>(ws + L.tab);
-      const size_t lds = (size_t)(MOE_ALIGN_WAVES + 2) * E * sizeof(int);
-      hipStream_t hs = (hipStream_t)stream;
-      hipLaunchKernelGGL(moe_align_count_kernel, dim3(parts), dim3(1024), lds, hs, ids, L.n_slots, E, part, tab);
-      hipLaunchKernelGGL(moe_align_scan_kernel, dim3(1), dim3(1024), (size_t)2 * E * sizeof(int), hs, L.n_slots, E,
-                         tile, L.cap, parts, tab, sorted, experts, npp);
-      hipLaunchKernelGGL(moe_align_place_kernel, dim3(parts), dim3(1024), lds, hs, ids, L.n_slots, E, part, tab,
-                         sorted);
-      st = launch_status();
-    } else {
-      st = awqmi_moe_align(ids, L.n_slots, E, tile, sorted, experts, npp, stream);
-    }
+    // long slot lists: count per part, scan, place per part (three launches, many workgroups)
+    if (const int rc = ensure_kernel_attributes()) return rc;
+    int parts = (L.n_slots + 4095) / 4096;
+    if (parts > MOE_ALIGN_PARTS_MAX) parts = MOE_ALIGN_PARTS_MAX;
+    const int part = ((L.n_slots + parts - 1) / parts + 63) / 64 * 64;
+    parts = (L.n_slots + part - 1) / part;
+    int32_t* tab = reinterpret_cast<int32_t*>(ws + L.tab);
+    const size_t lds = (size_t)(MOE_ALIGN_WAVES + 2) * E * sizeof(int);
+    hipStream_t hs = (hipStream_t)stream;
+    hipLaunchKernelGGL(moe_align_count_kernel, dim3(parts), dim3(1024), lds, hs, ids, L.n_slots, E, part, tab);
+    hipLaunchKernelGGL(moe_align_scan_kernel, dim3(1), dim3(1024), (size_t)2 * E * sizeof(int), hs, L.n_slots, E,
+                       tile, L.cap, parts, tab, sorted, experts, npp);
+    hipLaunchKernelGGL(moe_align_place_kernel, dim3(parts), dim3(1024), lds, hs, ids, L.n_slots, E, part, tab,
+                       sorted);
+    st = launch_status();
     if (st) return st;
   }
   const int Gn = norm_group(H, group);
@@ -974,11 +1039,11 @@ int awqmi_fused_moe_routed_f16(const void* hidden, const float* router_logits, c
     // the w13 GEMM writes silu(gate) * up itself: in one workgroup per gate / up block pair, or,
     // with few blocks (the launch is split in K), in the last arrivers of such a pair
     st = moe_gemm_impl(hidden, w13_q, w13_s, w13_z, act, sorted, experts, npp, nullptr, L.n_slots, topk, 16, E, H,
-                       2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream, true);
+                       2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream, true, pending);
     if (st) return st;
   } else {
-    st = awqmi_moe_gemm_f16(hidden, w13_q, w13_s, w13_z, h13, sorted, experts, npp, nullptr, L.n_slots, topk,
-                            tile, E, H, 2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream);
+    st = moe_gemm_impl(hidden, w13_q, w13_s, w13_z, h13, sorted, experts, npp, nullptr, L.n_slots, topk,
+                       tile, E, H, 2 * inter, group, 0, ws + L.gemm_ws, L.gemm_ws_bytes, stream, false, pending);
     if (st) return st;
     st = awqmi_silu_and_mul_f16(h13, act, L.n_slots, inter, stream);
     if (st) return st;

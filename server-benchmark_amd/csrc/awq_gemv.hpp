@@ -13,6 +13,7 @@
 // workgroup arrives last (arrival counter per column block, left at zero).
 #pragma once
 #include "awq_common.hpp"
+#include "awq_moe.hpp"
 
 #ifndef AWQMI_GEMV_WAVES_PER_SIMD
 #define AWQMI_GEMV_WAVES_PER_SIMD 1
@@ -46,6 +47,18 @@ struct GemvParams {
   int act_split; // split-K launch over [gate | up] columns: the last arriver of a gate block and
                  // its up block writes silu(gate) * up (one 16-row block, four waves per column block)
   long long w_stride, s_stride, z_stride;  // elements per expert
+  // Routing folded into the launch (ROUTE instantiations: at most eight tokens, 64 slots): every
+  // workgroup works the routing and the block list out by itself from the router logits, and
+  // the first workgroup also leaves them in memory for the launches that follow.
+  const float* r_logits;   // [r_T][r_E]
+  const float* r_bias;     // score-correction bias or null (sigmoid scoring)
+  int r_T, r_E, r_topk, r_renorm;
+  float r_scale;
+  int* r_ids;              // out [n_slots]
+  float* r_wts;            // out [n_slots]
+  int* r_sorted;           // out: 16 entries per block that runs
+  int* r_experts;          // out: one per block that runs
+  int* r_npp;              // out: 16 x blocks that run
 };
 
 typedef float f2 __attribute__((ext_vector_type(2)));
@@ -400,8 +413,19 @@ struct GemvWave {
 // LDSQ: weight ring of RING = 4 steps in LDS (see GemvWave), two workgroups per CU.
 // TAIL (dense launches, see GemvWave): every wave gets the same number of whole chunks and the
 // chunks left over are taken one 32-row step per wave.
-template <int WPL, int GMODE, int MB, bool MOE, int RING, int KW, bool ACT, bool LDSQ, bool TAIL>
+// RPER > 0 (MoE launches of a few tokens, at most 64 slots, 16-row blocks): the launch does its
+// own routing.  The four waves of EVERY workgroup run the top-k of the tokens in turn (RPER experts
+// per lane, RSIG = sigmoid scoring) into LDS; every wave then sorts the slots by expert in
+// registers (lane = slot: equal-expert mask from one ballot per id bit, block index = number of
+// distinct smaller experts) and so knows its block's expert and rows without a trip to memory.
+// A token picks distinct experts, so an expert holds at most T <= 8 slots and every block is one
+// expert's single block.  Workgroup 0 writes ids, weights, block list and padded count out for
+// the launches that follow (same layout as the align kernel's, entries past the last block that
+// runs left unwritten: nothing reads them).
+template <int WPL, int GMODE, int MB, bool MOE, int RING, int KW, bool ACT, bool LDSQ, bool TAIL, int RPER = 0,
+          bool RSIG = false>
 __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
+  static_assert(RPER == 0 || (MOE && MB == 1 && !TAIL), "folded routing: expert-grouped launches of 16-row blocks");
   static_assert(!ACT || (KW == 2 && MB == 1), "fused activation pairs two column blocks");
   static_assert(!LDSQ || (WPL == 2 && RING == 4), "the LDS ring holds four steps of 128-byte rows");
   static_assert(!TAIL || (!MOE && KW == 4 && !ACT), "tail steps are for dense launches");
@@ -440,15 +464,73 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
     blk = bg * B + slot % B;
     cb = cbs / p.split_k;          // column group of the workgroup (a column block when CW = 1)
     sp = cbs % p.split_k;
+    int e, sid = p.n_slots;
+    if constexpr (RPER > 0) {
+      __shared__ int r_ids_s[64];
+      __shared__ float r_wts_s[64];
+      __shared__ int r_stage[64 * 16];
+      __shared__ int r_exp_s[64];
+      const int n = p.n_slots;
+      for (int t = wave; t < p.r_T; t += 4)
+        moe_topk_token<RPER, RSIG>(p.r_logits, p.r_bias, t, p.r_E, p.r_topk, p.r_renorm, p.r_scale, r_ids_s,
+                                   r_wts_s);
+      __syncthreads();
+      const bool valid = lane < n;
+      const int e_i = valid ? r_ids_s[lane] : 0x7fffffff;
+      unsigned long long same = __ballot(valid);
+      const int nbits = 32 - __builtin_clz(max(p.r_E - 1, 1));
+      for (int b = 0; b < nbits; ++b) {
+        const bool bit = (e_i >> b) & 1;
+        const unsigned long long bal = __ballot(bit);
+        same &= bit ? bal : ~bal;
+      }
+      const int r_i = __popcll(same & ((1ull << lane) - 1ull));     // row inside the expert's block
+      const unsigned long long firsts = __ballot(valid && r_i == 0);
+      int b_i = 0;                                                  // block = distinct smaller experts
+      for (int jj = 0; jj < n; ++jj) {
+        const int ej = __builtin_amdgcn_readlane(e_i, jj);
+        if (((firsts >> jj) & 1ull) && ej < e_i) ++b_i;
+      }
+      const int nb = __popcll(firsts);
+      if (blockIdx.x == 0) {
+        // the lists for the launches that follow, staged in LDS so that pads and slots do not race
+        for (int i = tid; i < nb * 16; i += 256) r_stage[i] = n;
+        __syncthreads();
+        if (wave == 0 && valid) {
+          r_stage[b_i * 16 + r_i] = lane;
+          if (r_i == 0) r_exp_s[b_i] = e_i;
+        }
+        __syncthreads();
+        for (int i = tid; i < nb * 16; i += 256) p.r_sorted[i] = r_stage[i];
+        if (tid < nb) p.r_experts[tid] = r_exp_s[tid];
+        if (tid < n) {
+          p.r_ids[tid] = r_ids_s[tid];
+          p.r_wts[tid] = r_wts_s[tid];
+        }
+        if (tid == 0) p.r_npp[0] = nb * 16;
+      }
+      if (blk >= nb) return;
+      const unsigned long long mine = __ballot(valid && b_i == blk);
+      e = __builtin_amdgcn_readlane(e_i, __builtin_ctzll(mine));
+      // thread r takes the slot of row r: the r-th set lane of `mine` (at most eight rows)
+      unsigned long long m = mine;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        if (m) {
+          if (tid == k) sid = __builtin_ctzll(m);
+          m &= m - 1ull;
+        }
+      }
+    } else {
     // The block's padded count, expert and slot ids are read side by side (one trip to memory
     // instead of three in a row; blocks past the lists' end read the last block's entries and
     // leave right after), the routing weights behind them while the main loop runs.
     const int blk_c = min(blk, p.nblk_cap - 1);
     const int npp = *p.n_post_pad;
-    const int e = p.expert_ids[blk_c];
-    int sid = p.n_slots;
+    e = p.expert_ids[blk_c];
     if (tid < TM) sid = p.sorted_ids[blk_c * TM + tid];
     if (blk >= p.nblk_cap || blk * TM >= npp) return;
+    }
     qw += (size_t)e * p.w_stride;
     sc += (size_t)e * p.s_stride;
     qz += (size_t)e * p.z_stride;
@@ -746,6 +828,13 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
 template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false, bool LDSQ = false>
 __global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
   awq_gemv_body<WPL, GMODE, MB, MOE, RING, KW, ACT, LDSQ, false>(p);
+}
+
+// the expert-grouped launch of 16-row blocks (two words per lane, register ring of two) with the
+// routing folded in: RPER experts per lane, RSIG = sigmoid scoring
+template <int GMODE, int RPER, bool RSIG>
+__global__ __launch_bounds__(256, 2) void awq_gemv_route_kernel(const GemvParams p) {
+  awq_gemv_body<2, GMODE, 1, true, 2, 4, false, false, false, RPER, RSIG>(p);
 }
 
 // the dense G = 128 launch in its TAIL form (left-over chunks step by step)

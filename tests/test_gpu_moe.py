@@ -446,3 +446,51 @@ def test_fused_call_with_long_slot_lists(sba, gpu, T, E, topk):
     step = sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True, block_size=bs)
     assert torch.equal(one, step)
     assert torch.equal(one, sba.fused_moe_awq(c.x, c.w13, c.w2, c.logits, topk, True))
+
+
+@pytest.mark.parametrize("scoring", ["softmax", "sigmoid"])
+@pytest.mark.parametrize("T,H,E,topk,I", [(1, 2048, 128, 8, 768), (2, 2048, 128, 8, 768), (3, 2048, 128, 8, 768),
+                                          (4, 2048, 128, 8, 768), (4, 512, 64, 6, 256), (1, 256, 8, 1, 128),
+                                          (3, 1024, 16, 10, 512), (4, 256, 4, 4, 128), (2, 384, 100, 16, 128),
+                                          (4, 512, 128, 16, 256)])
+def test_routing_folded_into_the_first_expert_gemm(sba, gpu, scoring, T, H, E, topk, I):
+    """Blocks of at most four tokens (32 slots, 128 experts) have no routing launch: the first
+    expert GEMM works the routing out in every workgroup.  The result must have the bits of the
+    block with the routing launched on its own (development variant bit 1 << 24), also with
+    duplicate experts across tokens (few experts, large top-k), and must match the oracle's
+    forward with the oracle's routing."""
+    c = sba.workloads.make_moe_case(T, H, E, topk, I, 128, seed=11 * T + E)
+    cg = c.to(gpu)
+    kw = {}
+    bias = None
+    if scoring == "sigmoid":
+        bias = torch.randn((E,), generator=torch.Generator().manual_seed(E)) * 0.1
+        kw = dict(scoring_func="sigmoid", e_score_correction_bias=bias.to(gpu), routed_scaling_factor=1.25)
+    y = sba.fused_moe_awq(cg.x, cg.w13, cg.w2, cg.logits, topk, True, **kw).clone()
+    y_sep = sba.fused_moe_awq(cg.x, cg.w13, cg.w2, cg.logits, topk, True, _dev_variant=1 << 24, **kw).clone()
+    assert torch.equal(y.view(torch.int16), y_sep.view(torch.int16))
+    if scoring == "sigmoid":
+        ids, tw = awq_ref.topk_sigmoid(c.logits.numpy(), topk, True, bias.numpy(), 1.25)
+    else:
+        ids, tw = awq_ref.topk_softmax(c.logits.numpy(), topk, True)
+    ref = awq_ref.moe_forward(c.x.numpy(), tuple(a.numpy() for a in c.w13), tuple(a.numpy() for a in c.w2),
+                              ids, tw, 128)
+    assert awq_ref.rel_frobenius(y.cpu().numpy(), ref) <= TOL
+    # a second call on the same workspace, fewer tokens: nothing of the first call's lists is read
+    if T > 1:
+        y1 = sba.fused_moe_awq(cg.x[:1].contiguous(), cg.w13, cg.w2, cg.logits[:1].contiguous(), topk, True, **kw)
+        y1_sep = sba.fused_moe_awq(cg.x[:1].contiguous(), cg.w13, cg.w2, cg.logits[:1].contiguous(), topk, True,
+                                   _dev_variant=1 << 24, **kw)
+        assert torch.equal(y1.view(torch.int16), y1_sep.view(torch.int16))
+
+
+def test_folded_routing_with_nan_logits(sba, gpu):
+    """A NaN logit in a folded-routing block: ids stay in range (the block runs, every slot row is
+    written) and the output equals the separately routed block's, NaNs included."""
+    c = sba.workloads.make_moe_case(2, 512, 16, 4, 256, 128, seed=3).to(gpu)
+    lg = c.logits.clone()
+    lg[0, 3] = float("nan")
+    lg[1, :] = float("nan")
+    y = sba.fused_moe_awq(c.x, c.w13, c.w2, lg, 4, True).clone()
+    y_sep = sba.fused_moe_awq(c.x, c.w13, c.w2, lg, 4, True, _dev_variant=1 << 24).clone()
+    assert torch.equal(y.view(torch.int16), y_sep.view(torch.int16))
