@@ -255,7 +255,10 @@ static int ensure_kernel_attributes() {
       reinterpret_cast<const void*>(moe_align_count_kernel), reinterpret_cast<const void*>(moe_align_place_kernel),
       reinterpret_cast<const void*>(moe_route_align_kernel<1, false>), reinterpret_cast<const void*>(moe_route_align_kernel<2, false>),
       reinterpret_cast<const void*>(moe_route_align_kernel<4, false>), reinterpret_cast<const void*>(moe_route_align_kernel<8, false>),
-      reinterpret_cast<const void*>(moe_route_align_kernel<16, false>)};
+      reinterpret_cast<const void*>(moe_route_align_kernel<16, false>),
+      reinterpret_cast<const void*>(moe_route_align_kernel<1, true>), reinterpret_cast<const void*>(moe_route_align_kernel<2, true>),
+      reinterpret_cast<const void*>(moe_route_align_kernel<4, true>), reinterpret_cast<const void*>(moe_route_align_kernel<8, true>),
+      reinterpret_cast<const void*>(moe_route_align_kernel<16, true>)};
   for (const void* fn : align) {
     const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                              (MOE_ALIGN_WAVES + 2) * AWQMI_MAX_EXPERTS * (int)sizeof(int));
@@ -265,28 +268,36 @@ static int ensure_kernel_attributes() {
   return AWQMI_OK;
 }
 
-// softmax routing and align in one launch (at most 16 tokens); same results as the two calls
+// routing and align in one launch (at most 16 tokens); same results as the two calls
 template <int P>
-static int moe_route_align_launch(const float* logits, int T, int E, int topk, int renormalize,
-                                  int32_t* ids, float* wts, int tile_m, int cap, int32_t* sorted,
-                                  int32_t* experts, int32_t* npp, hipStream_t st) {
+static int moe_route_align_launch(const float* logits, const float* bias, int T, int E, int topk, int scoring,
+                                  int renormalize, float scale, int32_t* ids, float* wts, int tile_m, int cap,
+                                  int32_t* sorted, int32_t* experts, int32_t* npp, hipStream_t st) {
   if (const int rc = ensure_kernel_attributes()) return rc;
-  hipLaunchKernelGGL((moe_route_align_kernel<P, false>), dim3(1), dim3(1024),
-                     (size_t)(MOE_ALIGN_WAVES + 2) * E * sizeof(int), st, logits, (const float*)nullptr, T, E,
-                     topk, renormalize, 1.f, ids, wts, tile_m, cap, sorted, experts, npp);
+  const size_t lds = (size_t)(MOE_ALIGN_WAVES + 2) * E * sizeof(int);
+  if (scoring == 1)
+    hipLaunchKernelGGL((moe_route_align_kernel<P, true>), dim3(1), dim3(1024), lds, st, logits, bias, T, E, topk,
+                       renormalize, scale, ids, wts, tile_m, cap, sorted, experts, npp);
+  else
+    hipLaunchKernelGGL((moe_route_align_kernel<P, false>), dim3(1), dim3(1024), lds, st, logits, (const float*)nullptr,
+                       T, E, topk, renormalize, scale, ids, wts, tile_m, cap, sorted, experts, npp);
   return launch_status();
 }
 
-static int moe_route_align_small(const float* logits, int T, int E, int topk, int renormalize,
-                                 int32_t* ids, float* wts, int tile_m, int32_t* sorted, int32_t* experts,
-                                 int32_t* npp, void* stream) {
+static int moe_route_align_small(const float* logits, const float* bias, int T, int E, int topk, int scoring,
+                                 int renormalize, float scale, int32_t* ids, float* wts, int tile_m,
+                                 int32_t* sorted, int32_t* experts, int32_t* npp, void* stream) {
   const int cap = (int)awqmi_moe_align_capacity(T * topk, E, tile_m);
   hipStream_t st = (hipStream_t)stream;
-  if (E <= 64) return moe_route_align_launch<1>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
-  if (E <= 128) return moe_route_align_launch<2>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
-  if (E <= 256) return moe_route_align_launch<4>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
-  if (E <= 512) return moe_route_align_launch<8>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
-  return moe_route_align_launch<16>(logits, T, E, topk, renormalize, ids, wts, tile_m, cap, sorted, experts, npp, st);
+#define AWQMI_RA(P) \
+  return moe_route_align_launch<P>(logits, bias, T, E, topk, scoring, renormalize, scale, ids, wts, tile_m, cap, \
+                                   sorted, experts, npp, st)
+  if (E <= 64) AWQMI_RA(1);
+  if (E <= 128) AWQMI_RA(2);
+  if (E <= 256) AWQMI_RA(4);
+  if (E <= 512) AWQMI_RA(8);
+  AWQMI_RA(16);
+#undef AWQMI_RA
 }
 
 // Routing of one MoE block: inputs and the five lists it produces.
@@ -302,13 +313,12 @@ struct MoeRoute {
   int32_t* npp;
 };
 
-// Routing + align of a short slot list as launches of their own (one launch for plain softmax
-// routing of up to 16 tokens, else top-k and align apart).
+// Routing + align of a short slot list as launches of their own (one launch for up to 16
+// tokens, else top-k and align apart).
 static int moe_route_launches(const MoeRoute& r, int tile, void* stream) {
-  const bool plain = r.scoring == 0 && !r.bias && r.scale == 1.f;
-  if (r.T <= MOE_ALIGN_WAVES && plain)
-    return moe_route_align_small(r.logits, r.T, r.E, r.topk, r.renorm, r.ids, r.wts, tile, r.sorted, r.experts, r.npp,
-                                 stream);
+  if (r.T <= MOE_ALIGN_WAVES)
+    return moe_route_align_small(r.logits, r.bias, r.T, r.E, r.topk, r.scoring, r.renorm, r.scale, r.ids, r.wts, tile,
+                                 r.sorted, r.experts, r.npp, stream);
   if (const int st = awqmi_moe_topk_f32(r.logits, r.bias, r.T, r.E, r.topk, r.scoring, r.renorm, r.scale, r.ids, r.wts,
                                         stream))
     return st;
