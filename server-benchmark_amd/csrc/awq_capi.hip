@@ -124,8 +124,17 @@ inline bool gemv_tail_ok(int nchunks, int split) {
   return base >= 1 && left > 0 && 4 * left <= parts;
 }
 
-int pick_split_k(int rows, int K, int N, int G, long long blocks_z) {
-  (void)rows; (void)G;
+// dense launches of up to 16 rows with two words per lane and G = 128 can take the TAIL form
+inline bool gemv_tail_shape(int M, int N, int G) {
+  return M <= 16 && G == 128 && gemv_wpl(N) == 2 && !variant_on(VAR_NO_TAIL_STEP);
+}
+
+// dense: a dense launch (blocks_z = 1), which takes the TAIL form where its shape and the split
+// allow; the busiest wave is then counted in 32-row steps (on 21 layer shapes of eight model
+// sizes at 1 and 16 rows, every split forced in turn: the pick is the best split or within 2 % of
+// it on all 42 points; counting whole chunks was 6 - 8 % behind on the 5120-wide layers).
+int pick_split_k(int rows, int K, int N, int G, long long blocks_z, bool dense = false) {
+  const bool tail_form = dense && blocks_z == 1 && gemv_tail_shape(rows, N, G);
   const int nchunks = K / 128;
   const long long ncb = (N + 255) / 256;
   const long long wg = ncb * blocks_z;            // workgroups at split 1
@@ -138,9 +147,20 @@ int pick_split_k(int rows, int K, int N, int G, long long blocks_z) {
   double best_cost = 1e300;
   for (long long s = smax; s >= 1 && 2 * s >= smax; --s) {
     const long long parts = 4 * s;
-    const long long busiest = (nchunks + parts - 1) / parts;
     const double fill = (double)(wg * s) / 256.0;            // fraction of the round used
-    const double cost = (double)busiest * (double)parts / (double)nchunks / (0.5 + 0.5 * fill);
+    double cost;
+    if (tail_form) {
+      const long long steps = gemv_tail_ok(nchunks, (int)s) ? 4 * (nchunks / parts) + 1
+                                                            : 4 * ((nchunks + parts - 1) / parts);
+      // the finishing workgroup reads the parts eight at a time: every further batch is one more
+      // dependent trip to memory, over partial tiles that grow with the split
+      const double batches = (double)((s + 7) / 8 - 1);
+      cost = (double)steps * (double)parts / (4.0 * nchunks) / (0.4 + 0.6 * fill) * (1.0 + 0.15 * batches * batches);
+      if (cost <= best_cost + 1e-9) { best_cost = cost; best = s; }     // ties go to the smaller split
+      continue;
+    }
+    const long long busiest = (nchunks + parts - 1) / parts;
+    cost = (double)busiest * (double)parts / (double)nchunks / (0.5 + 0.5 * fill);
     if (cost < best_cost - 1e-9) { best_cost = cost; best = s; }
   }
   return (int)best;
@@ -150,11 +170,6 @@ inline size_t gemv_partial_bytes(int N, int split, long long blocks_z, int tile_
   if (split <= 1) return 0;
   const size_t npad = ((size_t)N + 255) / 256 * 256;
   return (size_t)split * (size_t)blocks_z * tile_m * npad * sizeof(float);
-}
-
-// dense launches of up to 16 rows with two words per lane and G = 128 can take the TAIL form
-inline bool gemv_tail_shape(int M, int N, int G) {
-  return M <= 16 && G == 128 && gemv_wpl(N) == 2 && !variant_on(VAR_NO_TAIL_STEP);
 }
 
 template <int WPL, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false, bool LDSQ = false>
@@ -405,7 +420,7 @@ int awqmi_gemm_auto_split_k(int M, int K, int N, int group) {
   const int G = norm_group(K, group);
   if (check_awq_shape(K, N, G) != AWQMI_OK || M <= 0) return 1;
   if (!skinny_rows(M, N) || !gemv_tiled_ok(K, G)) return 1;
-  return pick_split_k(M, K, N, G, 1);
+  return pick_split_k(M, K, N, G, 1, true);
 }
 
 size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
@@ -422,7 +437,8 @@ size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
   }
   if (M <= SKINNY_MAX_M) {
     int s = split_k;
-    if (s <= 0) s = (K % 128 == 0) ? pick_split_k(M, K, N, 128, 1) : 1;
+    // the pick depends on the group size (TAIL form only at G = 128): cover both
+    if (s <= 0) s = (K % 128 == 0) ? std::max(pick_split_k(M, K, N, 128, 1, true), pick_split_k(M, K, N, 64, 1, true)) : 1;
     skinny = gemv_partial_bytes(N, s, 1, 32);
   }
   return AWQMI_WS_COUNTER_BYTES + (mfma > skinny ? mfma : skinny);
@@ -456,7 +472,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   if (variant_on(VAR_MID_M_MFMA)) mid_skinny = false;
   if (gemv_tiled_ok(K, G) &&
       (M <= 16 || (M <= SKINNY_MAX_M && wpl == 2 && (mid_skinny || !mfma_ok)))) {
-    int split = split_k > 0 ? split_k : pick_split_k(M, K, N, G, 1);
+    int split = split_k > 0 ? split_k : pick_split_k(M, K, N, G, 1, true);
     const int nchunks = K / 128;
     if (split > nchunks) split = nchunks;
     const int ncb = (NW + 16 * wpl - 1) / (16 * wpl);
