@@ -343,9 +343,9 @@ static int moe_route_launches(const MoeRoute& r, int tile, void* stream) {
 // Folded routing: at most four tokens (one per wave of a workgroup; the kernel would take up to
 // eight in turn, but from five tokens on every workgroup spends on the second round what the
 // saved launch gains: 128 experts, top-8, weights from HBM: 3.5 us of 29 - 38 faster at 1 - 4
-// tokens, 0.9 us at 5, nothing at 6 - 8), 64 slots (one lane each), 128 experts (two per lane).
+// tokens, 0.9 us at 5, nothing at 6 - 8), 64 slots (one lane each), 256 experts (four per lane).
 static bool moe_route_foldable(int T, int E, int topk, int tile) {
-  return T <= 4 && T * topk <= 64 && E <= 128 && tile == 16 && !variant_on(VAR_NO_FOLDED_ROUTE);
+  return T <= 4 && T * topk <= 64 && E <= 256 && tile == 16 && !variant_on(VAR_NO_FOLDED_ROUTE);
 }
 
 extern "C" {
@@ -852,11 +852,16 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
       p.r_scale = route->scale;
       p.r_ids = route->ids; p.r_wts = route->wts; p.r_sorted = route->sorted; p.r_experts = route->experts;
       p.r_npp = route->npp;
-      const bool two = route->E > 64, sig = route->scoring == 1;
-      if (two && sig) hipLaunchKernelGGL((awq_gemv_route_kernel<2, 2, true>), grid, dim3(256), 0, st, p);
-      else if (two) hipLaunchKernelGGL((awq_gemv_route_kernel<2, 2, false>), grid, dim3(256), 0, st, p);
-      else if (sig) hipLaunchKernelGGL((awq_gemv_route_kernel<2, 1, true>), grid, dim3(256), 0, st, p);
-      else hipLaunchKernelGGL((awq_gemv_route_kernel<2, 1, false>), grid, dim3(256), 0, st, p);
+      const bool sig = route->scoring == 1;
+#define AWQMI_ROUTE(PERV)                                                                                   \
+  do {                                                                                                      \
+    if (sig) hipLaunchKernelGGL((awq_gemv_route_kernel<2, PERV, true>), grid, dim3(256), 0, st, p);        \
+    else hipLaunchKernelGGL((awq_gemv_route_kernel<2, PERV, false>), grid, dim3(256), 0, st, p);           \
+  } while (0)
+      if (route->E <= 64) AWQMI_ROUTE(1);
+      else if (route->E <= 128) AWQMI_ROUTE(2);
+      else AWQMI_ROUTE(4);
+#undef AWQMI_ROUTE
       return launch_status();
     }
     if (const int rc = moe_route_launches(*route, tile_m, stream)) return rc;

@@ -452,7 +452,7 @@ def test_fused_call_with_long_slot_lists(sba, gpu, T, E, topk):
 @pytest.mark.parametrize("T,H,E,topk,I", [(1, 2048, 128, 8, 768), (2, 2048, 128, 8, 768), (3, 2048, 128, 8, 768),
                                           (4, 2048, 128, 8, 768), (4, 512, 64, 6, 256), (1, 256, 8, 1, 128),
                                           (3, 1024, 16, 10, 512), (4, 256, 4, 4, 128), (2, 384, 100, 16, 128),
-                                          (4, 512, 128, 16, 256)])
+                                          (4, 512, 128, 16, 256), (2, 256, 160, 8, 128), (4, 256, 256, 8, 128)])
 def test_routing_folded_into_the_first_expert_gemm(sba, gpu, scoring, T, H, E, topk, I):
     """Blocks of at most four tokens (32 slots, 128 experts) have no routing launch: the first
     expert GEMM works the routing out in every workgroup.  The result must have the bits of the
