@@ -73,13 +73,20 @@ def make_weights(K, N, G, device, gen):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    # 50 untimed steps are 20 ms: with 5 (2 ms) the timed steps still ran 4 - 5 % slower than any later
+    # sweep of the same process (0.41 against 0.39 ms per step)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--launch", choices=("graph", "direct"), default="graph",
                     help="replay the step as a HIP graph (how a serving engine decodes) or launch directly")
     ap.add_argument("--split-k", type=int, default=0, help="0 = library heuristic")
     ap.add_argument("--variant", type=int, default=-1,
                     help="development: run the decode sweep through awqmi_dev_gemm_f16 with this launch-rule variant")
+    ap.add_argument("--rows", choices=("contiguous", "method"), default="contiguous",
+                    help="layout of the dense layers' qweight: contiguous as in the checkpoint (what the ops "
+                         "awq_gemm / awq_dequantize are handed by vLLM's own method), or as this package's "
+                         "AWQLinearMethod.process_weights_after_loading holds it (rows that are a multiple of "
+                         "1 KiB get one 128-byte line of pitch more); the other layout's sweep is timed beside it")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--decoder", action="store_true", help=argparse.SUPPRESS)   # kept for old command lines
@@ -98,6 +105,8 @@ def main():
                          "every weight, zero point, scale and activation (no operand bit toggles in the matrix pipe)")
     args = ap.parse_args()
 
+    if args.variant >= 0:
+        args.rows = "contiguous"      # the development entry point takes contiguous rows only
     if args.gpus != 1:
         log("bench.py: this build measures one GPU only: column-parallel layers shard the weight "
             "triple on N with no exchange, row-parallel layers shard K and add one all-reduce, "
@@ -128,8 +137,14 @@ def main():
     W = {}
     X = {}
     Y = {}
+    from server_benchmark_amd import ops
+
+    def held(triple):
+        qw, sc, qz = triple
+        return (ops.pad_qweight_rows(qw) if args.rows == "method" else qw), sc, qz
+
     for name, K, N in layers:
-        W[name] = [make_weights(K, N, G, dev, gen) for _ in range(NCOPY)]
+        W[name] = [held(make_weights(K, N, G, dev, gen)) for _ in range(NCOPY)]
         X[name] = {M: torch.randn((M, K), device=dev, generator=gen).to(torch.float16) for M in Ms}
         Y[name] = {M: torch.empty((M, N), dtype=torch.float16, device=dev) for M in Ms}
     ws_bytes = max(lib.awqmi_gemm_workspace_bytes(M, K, N, args.split_k) for _, K, N in layers
@@ -139,18 +154,21 @@ def main():
     log(f"[bench] inputs resident after {time.time() - t0:.1f}s, "
         f"{torch.cuda.memory_allocated() / 2**30:.2f} GiB allocated")
 
-    def launch(name, K, N, M, copy, stream_ptr):
-        qw, sc, qz = W[name][copy]
+    def launch(name, K, N, M, copy, stream_ptr, weights=None):
+        qw, sc, qz = (weights or W)[name][copy]
         a = (X[name][M].data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), Y[name][M].data_ptr(),
              ws.data_ptr(), ws.numel(), M, K, N, G, args.split_k, stream_ptr)
-        st = lib.awqmi_gemm_f16(*a) if args.variant < 0 else lib.awqmi_dev_gemm_f16(*a, args.variant)
+        if args.variant < 0:
+            st = lib.awqmi_gemm_ld_f16(a[0], a[1], qw.stride(0), *a[2:])
+        else:
+            st = lib.awqmi_dev_gemm_f16(*a, args.variant)
         if st != 0:
-            raise RuntimeError(f"awqmi_gemm_f16 failed: {lib.awqmi_status_string(st).decode()}")
+            raise RuntimeError(f"awq_gemm failed: {lib.awqmi_status_string(st).decode()}")
 
-    def step(stream_ptr):
+    def step(stream_ptr, weights=None):
         for ci, M in enumerate(Ms):
             for name, K, N in layers:
-                launch(name, K, N, M, ci, stream_ptr)
+                launch(name, K, N, M, ci, stream_ptr, weights)
 
     step_bytes = sum(workloads.linear_bytes(M, K, N, G) for _, K, N in layers for M in Ms)
     n_launch = len(layers) * len(Ms)
@@ -164,9 +182,9 @@ def main():
             xp.fill_(1.0)
         yp = torch.empty((8192, N), dtype=torch.float16, device=dev)
         for _ in range(3):
-            st = lib.awqmi_gemm_f16(xp.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), yp.data_ptr(),
-                                    ws.data_ptr(), ws.numel(), 8192, K, N, G, 0,
-                                    torch.cuda.current_stream().cuda_stream)
+            st = lib.awqmi_gemm_ld_f16(xp.data_ptr(), qw.data_ptr(), qw.stride(0), sc.data_ptr(), qz.data_ptr(),
+                                       yp.data_ptr(), ws.data_ptr(), ws.numel(), 8192, K, N, G, 0,
+                                       torch.cuda.current_stream().cuda_stream)
             assert st == 0
         torch.cuda.synchronize()
         log(f"[bench] pmc target: 3 x awq_gemm {name} M=8192 K={K} N={N} "
@@ -198,42 +216,66 @@ def main():
             f"4 device copies of {src.numel()} bytes")
         return
 
-    graph = None
-    if args.launch == "graph":
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            step(side.cuda_stream)          # warm the code objects outside capture
-        torch.cuda.current_stream().wait_stream(side)
+    def time_sweep(weights):
+        """W untimed steps, then exactly K timed ones; returns (wall seconds, event milliseconds)."""
+        graph = None
+        if args.launch == "graph":
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step(side.cuda_stream, weights)          # warm the code objects outside capture
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step(torch.cuda.current_stream().cuda_stream, weights)
+
+        def run_step():
+            if graph is not None:
+                graph.replay()
+            else:
+                step(torch.cuda.current_stream().cuda_stream, weights)
+
+        for _ in range(args.warmup):
+            run_step()
         torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            step(torch.cuda.current_stream().cuda_stream)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t_start = time.perf_counter()
+        e0.record()
+        for _ in range(args.steps):
+            run_step()
+        e1.record()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t_start, e0.elapsed_time(e1)
 
-    def run_step():
-        if graph is not None:
-            graph.replay()
-        else:
-            step(torch.cuda.current_stream().cuda_stream)
-
-    for _ in range(args.warmup):
-        run_step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t_start = time.perf_counter()
-    e0.record()
-    for _ in range(args.steps):
-        run_step()
-    e1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t_start
-    ev_ms = e0.elapsed_time(e1)
+    wall, ev_ms = time_sweep(None)
     ms_per_step = wall * 1e3 / args.steps
     value = step_bytes / (wall / args.steps) / 1e9
     kern_avg_us = ev_ms * 1e3 / (args.steps * n_launch)
     achieved = step_bytes / n_launch / (kern_avg_us * 1e-6) / 1e9
     log(f"[bench] decode sweep: {ms_per_step:.3f} ms/step wall, {ev_ms / args.steps:.3f} ms/step events, "
         f"{value:.0f} GB/s ({value / HBM_PEAK_GBS:.1%} of {HBM_PEAK_GBS:.0f})")
+
+    # the same sweep on the other qweight layout (only the layers whose rows the method pads differ)
+    other_rows = None
+    if args.variant < 0 and not args.sweep_only:
+        if args.rows == "method":
+            W_other = {n: [(qw.contiguous(), sc, qz) for qw, sc, qz in W[n]] for n in W}
+        else:
+            W_other = {n: [(ops.pad_qweight_rows(qw), sc, qz) for qw, sc, qz in W[n]] for n in W}
+        wall_o, ev_o = time_sweep(W_other)
+        wall_again, _ = time_sweep(None)       # the headline layout once more, right behind it (clock drift)
+        other_rows = {"rows": ("contiguous" if args.rows == "method" else
+                               "as AWQLinearMethod.process_weights_after_loading holds them (qkv / o / down rows "
+                               "one 128-byte line further apart)"),
+                      "value": round(step_bytes / (wall_o / args.steps) / 1e9, 1), "unit": "GB/s",
+                      "ms_per_step": round(wall_o * 1e3 / args.steps, 4),
+                      "frac_hbm": round(step_bytes / (wall_o / args.steps) / 1e9 / HBM_PEAK_GBS, 4),
+                      "headline_layout_retimed_GBps": round(step_bytes / (wall_again / args.steps) / 1e9, 1)}
+        log(f"[bench] the same sweep with the other qweight row layout ({'contiguous' if args.rows == 'method' else 'method'}): "
+            f"{other_rows['ms_per_step']:.3f} ms/step, {other_rows['value']:.0f} GB/s; headline layout again: "
+            f"{other_rows['headline_layout_retimed_GBps']:.0f} GB/s")
+        del W_other
 
     if args.sweep_only:
         args.no_prefill = args.no_cpu = True
@@ -283,7 +325,12 @@ def main():
         "config": {"workload": "decode GEMV sweep, Qwen2.5-72B AWQ layer shapes (qkv 8192x10240, o 8192x8192, "
                                "gate_up 8192x59136, down 29568x8192), group 128, M in {1,4,8,16}; "
                                "16 awq_gemm launches per step, 4 rotating weight copies per layer",
-                   "launch": args.launch, "split_k": args.split_k, "bytes_per_step": step_bytes},
+                   "launch": args.launch, "split_k": args.split_k, "bytes_per_step": step_bytes,
+                   "qweight_rows": ("as AWQLinearMethod.process_weights_after_loading holds them: int32 [K, N/8] "
+                                    "with the rows of qkv / o / down (multiples of 1 KiB) one 128-byte line further "
+                                    "apart, values and shapes unchanged, pad never read"
+                                    if args.rows == "method" else "contiguous, as in the checkpoint")},
+        "other_qweight_rows": other_rows,
         "peaks": {"hbm_GBps": HBM_PEAK_GBS, "hbm_source": "MI355X published HBM3E bandwidth, 8 TB/s",
                   "mfma_fp16_TFLOPs": MFMA_FP16_PEAK_TFLOPS,
                   "mfma_source": "256 CUs x 4096 fp16 flop/clk/CU (dense MFMA) x 2.4 GHz = 2516.6 TFLOP/s, "
@@ -310,8 +357,8 @@ def main():
                 y = torch.empty((M, N), dtype=torch.float16, device=dev)
 
                 def call():
-                    st = lib.awqmi_gemm_f16(x.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(),
-                                            y.data_ptr(), ws.data_ptr(), ws.numel(), M, K, N, G, 0, stream_ptr)
+                    st = lib.awqmi_gemm_ld_f16(x.data_ptr(), qw.data_ptr(), qw.stride(0), sc.data_ptr(), qz.data_ptr(),
+                                               y.data_ptr(), ws.data_ptr(), ws.numel(), M, K, N, G, 0, stream_ptr)
                     if st != 0:
                         raise RuntimeError(lib.awqmi_status_string(st).decode())
 
@@ -349,8 +396,8 @@ def main():
             o = torch.empty((K, N), dtype=torch.float16, device=dev)
 
             def call():
-                st = lib.awqmi_dequantize_f16(qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), o.data_ptr(), K, N, G,
-                                              stream_ptr)
+                st = lib.awqmi_dequantize_ld_f16(qw.data_ptr(), qw.stride(0), sc.data_ptr(), qz.data_ptr(), o.data_ptr(),
+                                                 K, N, G, stream_ptr)
                 if st != 0:
                     raise RuntimeError(lib.awqmi_status_string(st).decode())
 

@@ -41,7 +41,7 @@ typedef enum awqmi_status {
   AWQMI_SCRATCH_LIMIT = 8        /* awqmi_gemm_f16_noalloc: needs > AWQMI_STATIC_SCRATCH_BYTES */
 } awqmi_status;
 
-#define AWQMI_VERSION 200        /* major*10000 + minor*100 + patch */
+#define AWQMI_VERSION 201        /* major*10000 + minor*100 + patch */
 #define AWQMI_MOE_TILE_M 16      /* default rows per sorted-token block (32 also accepted)  */
 #define AWQMI_MAX_SPLIT_K 64
 #define AWQMI_MAX_EXPERTS 1024
@@ -93,6 +93,21 @@ size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k);
 int awqmi_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
                    const int32_t* qzeros, void* y_f16, void* workspace, size_t workspace_bytes,
                    int M, int K, int N, int group, int split_k, void* stream);
+
+/* awqmi_gemm_f16 / awqmi_dequantize_f16 on a qweight whose rows are ldw int32 words apart in
+ * memory (ldw == N / 8, or larger and a multiple of 4; the words past N / 8 of a row are never read).  This is
+ * the form AWQLinearMethod.process_weights_after_loading hands over: vLLM's quantisation
+ * methods re-lay their weights out for their kernels in that hook (reached when the server of
+ * reference utils/generate_compose.py:85-93 loads a checkpoint), and this library's re-layout is
+ * a row pitch that is not a multiple of eight 128-byte lines -- with such a pitch the skinny
+ * kernel streams 12 - 20 % faster (every wave reads one line per row, and rows a multiple of
+ * 1 KiB apart put all of a wave's requests on the same address bits 7 - 9).  qzeros and scales
+ * stay contiguous.  With ldw == N / 8 these are awqmi_gemm_f16 / awqmi_dequantize_f16. */
+int awqmi_gemm_ld_f16(const void* x_f16, const int32_t* qweight, int ldw, const void* scales_f16,
+                      const int32_t* qzeros, void* y_f16, void* workspace, size_t workspace_bytes,
+                      int M, int K, int N, int group, int split_k, void* stream);
+int awqmi_dequantize_ld_f16(const int32_t* qweight, int ldw, const void* scales_f16,
+                            const int32_t* qzeros, void* out_f16, int K, int N, int group, void* stream);
 
 /* awqmi_gemm_f16 for callers that cannot allocate or carry a workspace: code under HIP graph
  * capture that has no buffer of its own, tight serving loops, harnesses that forbid hipMalloc.

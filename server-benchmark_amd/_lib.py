@@ -21,6 +21,10 @@ SIGNATURES = {
     "awqmi_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "awqmi_gemm_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "awqmi_gemm_ld_f16": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                  c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "awqmi_dequantize_ld_f16": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                        c_void_p]),
     "awqmi_gemm_f16_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                        c_int, c_void_p]),
     "awqmi_moe_topk_softmax_f32": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),

@@ -389,9 +389,15 @@ int awqmi_last_hip_error(void) { return t_last_hip_error; }
 
 int awqmi_dequantize_f16(const int32_t* qweight, const void* scales, const int32_t* qzeros,
                          void* out, int K, int N, int group, void* stream) {
+  return awqmi_dequantize_ld_f16(qweight, N / 8, scales, qzeros, out, K, N, group, stream);
+}
+
+int awqmi_dequantize_ld_f16(const int32_t* qweight, int ldw, const void* scales, const int32_t* qzeros,
+                            void* out, int K, int N, int group, void* stream) {
   if (!qweight || !scales || !qzeros || !out) return AWQMI_NULL_POINTER;
   const int G = norm_group(K, group);
   if (const int rc = check_awq_shape(K, N, G)) return rc;
+  if (ldw < N / 8 || (ldw != N / 8 && ldw % 4 != 0)) return AWQMI_BAD_ARGUMENT;
   if (!aligned16(scales) || !aligned16(out) || !aligned16(qweight) || !aligned16(qzeros))
     return AWQMI_BAD_ALIGN;
   const int NW = N / 8;
@@ -405,7 +411,7 @@ int awqmi_dequantize_f16(const int32_t* qweight, const void* scales, const int32
   for (int k0 = 0; k0 < K; k0 += 65535 * R) {                                                    \
     const int slabs = (K - k0) / R < 65535 ? (K - k0) / R : 65535;                               \
     hipLaunchKernelGGL((awq_dequant_kernel<R>), dim3(gx, slabs), dim3(256), 0, st, qw, sc, qz, o, k0, \
-                       NW, G);                                                                   \
+                       NW, G, ldw);                                                              \
   }
   if (G % 16 == 0) AWQMI_DQ(16)
   else if (G % 8 == 0) AWQMI_DQ(8)
@@ -447,11 +453,19 @@ size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
 int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
                    void* y, void* workspace, size_t workspace_bytes, int M, int K, int N, int group,
                    int split_k, void* stream) {
+  return awqmi_gemm_ld_f16(x, qweight, N / 8, scales, qzeros, y, workspace, workspace_bytes, M, K, N, group, split_k,
+                           stream);
+}
+
+int awqmi_gemm_ld_f16(const void* x, const int32_t* qweight, int ldw, const void* scales, const int32_t* qzeros,
+                      void* y, void* workspace, size_t workspace_bytes, int M, int K, int N, int group,
+                      int split_k, void* stream) {
   if (!x || !qweight || !scales || !qzeros || !y) return AWQMI_NULL_POINTER;
   const int G = norm_group(K, group);
   if (const int rc = check_awq_shape(K, N, G)) return rc;
   if (M <= 0) return AWQMI_BAD_SHAPE;
   if (split_k < 0 || split_k > AWQMI_MAX_SPLIT_K) return AWQMI_BAD_ARGUMENT;
+  if (ldw < N / 8 || (ldw != N / 8 && ldw % 4 != 0)) return AWQMI_BAD_ARGUMENT;
   if (!aligned16(x) || !aligned16(scales) || !aligned16(qweight) || !aligned16(qzeros) ||
       !aligned16(y))
     return AWQMI_BAD_ALIGN;
@@ -465,7 +479,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
 
   const int wpl = gemv_wpl(N);
   const bool mfma_ok = K % PF_BK == 0 && (((G & (G - 1)) == 0 && G >= 8) || G % 64 == 0) &&
-                       mfma_slab_rows(M, K) > 0 && (size_t)K * NW * 4 < (1ull << 32) &&
+                       mfma_slab_rows(M, K) > 0 && (size_t)K * ldw * 4 < (1ull << 32) &&
                        (size_t)(K / G) * N * 2 < (1ull << 32);
   bool mid_skinny = skinny_rows(M, N);
   if (variant_on(VAR_MID_M_SKINNY)) mid_skinny = true;
@@ -488,7 +502,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
     p.cnt = reinterpret_cast<int*>(workspace);
     p.part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
                        : nullptr;
-    p.K = K; p.N = N; p.NW = NW; p.G = G; p.ldy = N;
+    p.K = K; p.N = N; p.NW = NW; p.ldw = ldw; p.G = G; p.ldy = N;
     p.split_k = split; p.ncb = ncb;
     const dim3 grid(ncb, split, 1);
     // passes of up to 32 rows; each pass streams the weights once
@@ -499,7 +513,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
       // 17 .. 32 rows with long wave ranges (six chunks or more): the weight ring in LDS leaves the
       // register file to the two accumulator sets (gate_up / down_proj of the 72B shapes 3 - 11 %
       // faster, bit-identical; short ranges measured equal or 1 - 2 % slower)
-      const bool lds32 = nchunks >= 24 * split && (size_t)K * NW * 4 < (1ull << 31) && !variant_on(VAR_NO_LDS_RING);
+      const bool lds32 = nchunks >= 24 * split && (size_t)K * ldw * 4 < (1ull << 31) && !variant_on(VAR_NO_LDS_RING);
       if (p.M > 16 && lds32) launch_gemv<2, 2, false, 4, 4, false, true>(p, grid, st);
       else if (p.M > 16) launch_gemv<2, 2, false>(p, grid, st);
       else if (gemv_tail_shape(p.M, N, G) && gemv_tail_ok(nchunks, split))
@@ -520,7 +534,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
       const int Ms = M - r0 < slab ? M - r0 : slab;
       MfmaGemmParams p{};
       p.x = xx + (size_t)r0 * K; p.qw = qw; p.sc = sc; p.qz = qz; p.y = yy + (size_t)r0 * N;
-      p.M = Ms; p.K = K; p.N = N; p.NW = NW; p.G = G;
+      p.M = Ms; p.K = K; p.N = N; p.NW = NW; p.ldw = ldw; p.G = G;
       p.gshift = 0;
       if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
       int mi = mfma_pick_rows(Ms, K, N) / 64;
@@ -568,7 +582,7 @@ int awqmi_gemm_f16(const void* x, const int32_t* qweight, const void* scales, co
   for (int r0 = 0; r0 < M; r0 += 32768) {
     const int Ms = M - r0 < 32768 ? M - r0 : 32768;
     hipLaunchKernelGGL(awq_gemm_generic_kernel, dim3((NW + 255) / 256, Ms), dim3(256), 0, st,
-                       xx + (size_t)r0 * K, qw, sc, qz, yy + (size_t)r0 * N, Ms, K, NW, G);
+                       xx + (size_t)r0 * K, qw, sc, qz, yy + (size_t)r0 * N, Ms, K, NW, G, ldw);
   }
   return launch_status();
 }
@@ -759,7 +773,7 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
     p.sc = reinterpret_cast<const half_t*>(scales);
     p.qz = reinterpret_cast<const uint32_t*>(qzeros);
     p.y = reinterpret_cast<half_t*>(y);
-    p.M = (int)x_rows; p.K = K; p.N = N; p.NW = NW; p.G = G;
+    p.M = (int)x_rows; p.K = K; p.N = N; p.NW = NW; p.ldw = NW; p.G = G;
     const bool pow2g = (G & (G - 1)) == 0 && G >= 8;
     p.gshift = 0;
     if (pow2g) while ((1 << p.gshift) < G) ++p.gshift;
@@ -802,7 +816,7 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   p.cnt = reinterpret_cast<int*>(workspace);
   p.part = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES)
                      : nullptr;
-  p.M = tile_m; p.K = K; p.N = N; p.NW = NW; p.G = G;
+  p.M = tile_m; p.K = K; p.N = N; p.NW = NW; p.ldw = NW; p.G = G;
   p.split_k = split; p.ncb = ncb;
   p.sorted_ids = sorted_token_ids; p.expert_ids = expert_ids; p.n_post_pad = num_tokens_post_padded;
   p.topk_w = topk_weights; p.n_slots = n_slots; p.a_row_div = a_row_div; p.tile_m = tile_m;

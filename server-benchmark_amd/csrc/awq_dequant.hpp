@@ -29,7 +29,7 @@ __global__ __launch_bounds__(256) void awq_dequant_kernel(const uint32_t* __rest
                                                           const half_t* __restrict__ sc,
                                                           const uint32_t* __restrict__ qz,
                                                           half_t* __restrict__ out, int k_base,
-                                                          int NW, int G) {
+                                                          int NW, int G, int ldw) {
   const int wc = blockIdx.x * 256 + threadIdx.x;
   if (wc >= NW) return;
   const size_t N = (size_t)NW * 8;
@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256) void awq_dequant_kernel(const uint32_t* __rest
   for (int j = 0; j < 4; ++j) zz[j] = ((z >> (4 * j)) & MASK_LO) | MAGIC_LO;
   uint32_t q[ROWS];
 #pragma unroll
-  for (int r = 0; r < ROWS; ++r) q[r] = __builtin_nontemporal_load(qw + (size_t)(k0 + r) * NW + wc);
+  for (int r = 0; r < ROWS; ++r) q[r] = __builtin_nontemporal_load(qw + (size_t)(k0 + r) * ldw + wc);
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
     const u4v o = dequant_word(q[r], zz, s);
@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256) void awq_gemm_generic_kernel(const half_t* __r
                                                                const half_t* __restrict__ sc,
                                                                const uint32_t* __restrict__ qz,
                                                                half_t* __restrict__ y, int M, int K,
-                                                               int NW, int G) {
+                                                               int NW, int G, int ldw) {
   const int wc = blockIdx.x * 256 + threadIdx.x;
   const int m = blockIdx.y;
   if (wc >= NW || m >= M) return;
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void awq_gemm_generic_kernel(const half_t* __r
 #pragma unroll
       for (int j = 0; j < 4; ++j) zz[j] = ((z >> (4 * j)) & MASK_LO) | MAGIC_LO;
     }
-    const u4v w = dequant_word(qw[(size_t)k * NW + wc], zz, s);
+    const u4v w = dequant_word(qw[(size_t)k * ldw + wc], zz, s);
     const float xv = (float)x[(size_t)m * K + k];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {

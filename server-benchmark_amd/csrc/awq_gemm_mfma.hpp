@@ -33,6 +33,7 @@ struct MfmaGemmParams {
   const uint32_t* qz;
   half_t* y;
   int M, K, N, NW, G;
+  int ldw;        // words between consecutive rows of qweight (NW, or more when the rows are padded)
   int gshift;     // log2(G) when G is a power of two (kernel instantiation POW2G)
   int mt, nt;     // tile counts
   int total;      // mt * nt
@@ -150,7 +151,7 @@ __global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const 
   const int wm = (wave / (NWV / 2)) * (32 * MI), wn = (wave % (NWV / 2)) * (32 * NJ);
 
   const __amdgpu_buffer_rsrc_t rx = pf_rsrc(p.x, (size_t)p.M * p.K * 2);
-  const __amdgpu_buffer_rsrc_t rw = pf_rsrc(qw_base, (size_t)p.K * p.NW * 4);
+  const __amdgpu_buffer_rsrc_t rw = pf_rsrc(qw_base, (size_t)p.K * p.ldw * 4);
   const __amdgpu_buffer_rsrc_t rz = pf_rsrc(qz_base, (size_t)(p.K / p.G) * p.NW * 4);
   const __amdgpu_buffer_rsrc_t rs = pf_rsrc(sc_base, (size_t)(p.K / p.G) * p.N * 2);
 
@@ -177,8 +178,9 @@ __global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const 
   const int kk = tid >> 5, wcl = tid & 31;
   int wcg = n0 / 8 + wcl;
   if (wcg >= p.NW) wcg = 0;                      // columns never stored; keep loads in bounds
-  const uint32_t w_off = (uint32_t)(((size_t)RW * kk * p.NW + wcg) * 4);
-  const uint32_t row_b = (uint32_t)p.NW * 4;     // bytes between qweight / qzeros rows
+  const uint32_t w_off = (uint32_t)(((size_t)RW * kk * p.ldw + wcg) * 4);
+  const uint32_t row_w = (uint32_t)p.ldw * 4;    // bytes between qweight rows
+  const uint32_t row_b = (uint32_t)p.NW * 4;     // bytes between qzeros rows
   const int b_t = (RW == 8 ? kk : (kk >> 1)) ^ (wcl & 7);   // physical 16-byte slot of column c: b_t ^ c
   const int b_half = RW == 8 ? 0 : (kk & 1) * 8;            // 8-byte half of the slot (RW = 4)
   const int b_base = wcl * 8 * PF_ROW_BYTES;
@@ -218,10 +220,10 @@ __global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const 
     for (int i = 0; i < AL; ++i) areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, a_off[i], so, 0);
   };
   auto gload_w = [&](int kt, int set) {
-    const uint32_t so = (uint32_t)kt * PF_BK * row_b;
+    const uint32_t so = (uint32_t)kt * PF_BK * row_w;
 #pragma unroll
     for (int i = 0; i < RW; ++i)
-      wreg[set][i] = __builtin_amdgcn_raw_buffer_load_b32(rw, w_off, so + i * row_b, 0);
+      wreg[set][i] = __builtin_amdgcn_raw_buffer_load_b32(rw, w_off, so + i * row_w, 0);
     if (POW2G) {
       const uint32_t g = (uint32_t)(kt * PF_BK + RW * kk) >> p.gshift;
       zreg[set] = __builtin_amdgcn_raw_buffer_load_b32(rz, g * row_b + wcg * 4, 0, 0);

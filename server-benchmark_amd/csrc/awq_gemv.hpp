@@ -30,6 +30,7 @@ struct GemvParams {
   float* part;  // [split][nblk*ncb][16][128*WPL] fp32 partial tiles (tile-major columns)
   int* cnt;     // [nblk*ncb] arrival counters
   int M, K, N, NW, G;
+  int ldw;      // words between consecutive rows of qweight (NW, or more when the rows are padded)
   int split_k;
   int ncb;      // column blocks
   // expert-grouped launch
@@ -139,10 +140,10 @@ struct GemvWave {
 
   const uint32_t* qw_u;      // wave-uniform base of the expert's qweight
   const half_t* x_lane[MB];  // this lane's activation row per row block, 8h applied
-  uint32_t q_off;            // this lane's byte offset inside a 32-row step: (8h * NW + wc) * 4
+  uint32_t q_off;            // this lane's byte offset inside a 32-row step: (8h * LDW + wc) * 4
   const half_t* sc;          // lane's scale pointer (8 * wc applied)
   const uint32_t* qz;        // lane's zero-word pointer (wc applied)
-  int NW, N, kspg, ngroups;  // kspg: 32-row steps per quantisation group
+  int NW, LDW, N, kspg, ngroups;  // LDW: words between qweight rows; kspg: 32-row steps per quantisation group
 
   qvec q[LDSQ ? 2 : RING][8];   // LDSQ: the step being computed and the next one, read from the LDS ring
   u4v a[RING][MB];
@@ -164,18 +165,18 @@ struct GemvWave {
     if constexpr (LDSQ) {
 #if defined(__HIP_DEVICE_COMPILE__)
       typedef __attribute__((address_space(3))) void lds_void;
-      const uint32_t so = (uint32_t)ks * 32u * (uint32_t)NW * 4u;
+      const uint32_t so = (uint32_t)ks * 32u * (uint32_t)LDW * 4u;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rq, (lds_void*)(slot[d] + i * 1024), 16, dma_v[i & 1],
-                                                 so + (uint32_t)i * 8u * (uint32_t)NW * 4u, 0, 0);
+                                                 so + (uint32_t)i * 8u * (uint32_t)LDW * 4u, 0, 0);
 #endif
     } else {
-      const char* rowbase = reinterpret_cast<const char*>(qw_u) + (size_t)ks * 32 * NW * 4;
+      const char* rowbase = reinterpret_cast<const char*>(qw_u) + (size_t)ks * 32 * LDW * 4;
 #pragma unroll
       for (int i = 0; i < 8; ++i)
         q[d][i] = __builtin_nontemporal_load(
-            reinterpret_cast<const qvec*>(rowbase + (size_t)i * NW * 4 + q_off));
+            reinterpret_cast<const qvec*>(rowbase + (size_t)i * LDW * 4 + q_off));
     }
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -572,19 +573,20 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
     unsigned char* const slots[4] = {lq0, lq1, lq2, lq3};
 #pragma unroll
     for (int d = 0; d < RING; ++d) w.slot[d] = slots[d] + wave_u * 4096;
-    w.rq = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(qw), 0, (int)((size_t)p.K * p.NW * 4), 0x00020000);
+    w.rq = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(qw), 0, (int)((size_t)p.K * p.ldw * 4), 0x00020000);
     const int wc4 = cbw * (16 * WPL) + 4 * (lane & 7);       // first of the four words this lane fetches
     // line 8 i + l / 8 of the slot (instruction i, lane l) holds row 8 i + ((l / 8) ^ (i & 1))
-    w.dma_v[0] = (uint32_t)(((size_t)(lane >> 3) * p.NW + (wc4 < p.NW ? wc4 : 0)) * 4);
-    w.dma_v[1] = (uint32_t)(((size_t)((lane >> 3) ^ 1) * p.NW + (wc4 < p.NW ? wc4 : 0)) * 4);
+    w.dma_v[0] = (uint32_t)(((size_t)(lane >> 3) * p.ldw + (wc4 < p.NW ? wc4 : 0)) * 4);
+    w.dma_v[1] = (uint32_t)(((size_t)((lane >> 3) ^ 1) * p.ldw + (wc4 < p.NW ? wc4 : 0)) * 4);
     // row 8 h + i is read from line 8 h + (i ^ (h & 1))
     w.rd_off[0] = (uint32_t)((8 * h + (h & 1)) * 128 + 8 * j);
     w.rd_off[1] = (uint32_t)((8 * h + (1 ^ (h & 1))) * 128 + 8 * j);
   }
-  w.q_off = (uint32_t)(((size_t)8 * h * p.NW + wc) * 4);
+  w.q_off = (uint32_t)(((size_t)8 * h * p.ldw + wc) * 4);
   w.sc = sc + 8 * (size_t)wc;
   w.qz = qz + wc;
   w.NW = p.NW;
+  w.LDW = p.ldw;
   w.N = p.N;
   w.kspg = p.G / 32;
   w.ngroups = GMODE == 3 ? p.K / p.G : p.K >> (5 + GMODE);

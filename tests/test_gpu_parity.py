@@ -411,3 +411,72 @@ def test_gemm_random_shapes_across_dispatch_boundaries(sba, gpu):
         assert err <= TOL, f"M={M} K={K} N={N} G={G}: rel_fro={err:.3e}"
         worst = max(worst, err)
     print(f"[random shapes] worst rel_fro={worst:.2e}", flush=True)
+
+
+def _with_pitch(qw_dev, extra_words):
+    """The same qweight as a view of a buffer whose rows are extra_words further apart; the pad
+    holds a pattern that would show up in the result if it were ever read."""
+    K, NW = qw_dev.shape
+    width = (NW + extra_words + 3) // 4 * 4          # a row pitch must keep 16-byte groups whole
+    buf = torch.full((K, width), 0x5A5A5A5A, dtype=torch.int32, device=qw_dev.device)
+    v = buf[:, :NW]
+    v.copy_(qw_dev)
+    return v
+
+
+@pytest.mark.parametrize("M,K,N,G,pitch,split", [
+    (1, 1024, 2048, 128, 32, 0), (16, 1024, 2048, 128, 32, 0), (5, 4096, 2048, 128, 32, 3),     # skinny, tail form
+    (16, 2048, 264, 64, 4, 0), (3, 512, 136, 256, 12, 2), (7, 256, 8, 32, 36, 0),                 # other groups, one word per lane
+    (24, 12288, 512, 128, 32, 0), (32, 3072, 2048, 64, 32, 1), (48, 1024, 2048, 128, 32, 0),    # 32-row passes, LDS ring
+    (64, 512, 2048, 128, 32, 0), (100, 1024, 520, 128, 8, 0), (300, 2048, 2048, 128, 32, 0),    # MFMA tiles
+    (700, 1024, 2064, 32, 4, 0), (512, 1024, 4096, 128, 32, 0),
+    (3, 96, 40, 32, 4, 0), (20, 100, 16, 50, 8, 0)])                                              # generic kernel
+def test_qweight_with_a_row_pitch(sba, gpu, M, K, N, G, pitch, split):
+    """qweight rows `pitch` words further apart than a row is long (what
+    AWQLinearMethod.process_weights_after_loading hands over for rows that are a multiple of 1 KiB):
+    awq_gemm on every kernel and awq_dequantize give the bits of the contiguous tensor, and match
+    the oracle; the pad is never read."""
+    x, qw, s, qz = _np_case(M, K, N, G, seed=M + K + N)
+    g = K if G <= 0 else G
+    xd, qwd, sd, qzd = _dev(gpu, x, qw, s, qz)
+    qwp = _with_pitch(qwd, pitch)
+    assert not qwp.is_contiguous() and qwp.stride(0) >= N // 8 + pitch
+    y0 = sba.awq_gemm(xd, qwd, sd, qzd, force_split_k=split)
+    y1 = sba.awq_gemm(xd, qwp, sd, qzd, force_split_k=split)
+    assert torch.equal(y0.view(torch.int16), y1.view(torch.int16))
+    ref = awq_ref.gemm_wide(x, qw, s, qz, g)
+    assert awq_ref.rel_frobenius(y1.cpu().numpy(), ref) <= TOL
+    W0 = sba.awq_dequantize(qwd, sd, qzd)
+    W1 = sba.awq_dequantize(qwp, sd, qzd)
+    assert torch.equal(W0.view(torch.int16), W1.view(torch.int16))
+    Wref = awq_ref.dequantize(qw, s, qz, g)
+    assert np.array_equal(W1.cpu().numpy().view(np.uint16), Wref.view(np.uint16))
+
+
+def test_qweight_pitch_is_validated(sba, gpu):
+    x, qw, s, qz = _np_case(4, 256, 256, 128, seed=1)
+    xd, qwd, sd, qzd = _dev(gpu, x, qw, s, qz)
+    bad = torch.zeros((256, 34), dtype=torch.int32, device=gpu)[:, :32]      # pitch not a multiple of 4 words
+    with pytest.raises(ValueError):
+        sba.awq_gemm(xd, bad, sd, qzd)
+    with pytest.raises(ValueError):
+        sba.awq_gemm(xd, qwd.t().contiguous().t(), sd, qzd)      # column-major
+
+
+def test_linear_method_pads_kib_rows_and_matches_contiguous(sba, gpu):
+    """A layer whose packed rows are 1 KiB: process_weights_after_loading re-pitches qweight, apply
+    gives the bits of awq_gemm on the contiguous tensor at decode and prefill sizes."""
+    cfg = sba.AWQConfig(4, 128, True)
+    m = sba.AWQLinearMethod(cfg)
+    layer = torch.nn.Module()
+    m.create_weights(layer, 1024, [2048], 1024, 2048, torch.float16, device=gpu)
+    x, qw, s, qz = _np_case(300, 1024, 2048, 128, seed=77)
+    layer.load_state_dict({"qweight": torch.from_numpy(qw), "qzeros": torch.from_numpy(qz),
+                           "scales": torch.from_numpy(s)})
+    m.process_weights_after_loading(layer)
+    assert layer.qweight.stride() == (288, 1)
+    xd, qwd, sd, qzd = _dev(gpu, x, qw, s, qz)
+    for rows in (1, 16, 40, 300):
+        y = m.apply(layer, xd[:rows].contiguous())
+        y0 = sba.awq_gemm(xd[:rows].contiguous(), qwd, sd, qzd)
+        assert torch.equal(y.view(torch.int16), y0.view(torch.int16))

@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol(lib):
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
     assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
-    assert lib.awqmi_version() == 200
+    assert lib.awqmi_version() == 201
 
 
 def test_status_strings(lib):
@@ -105,6 +105,43 @@ def test_workspace_reset_and_dev_entry_points_validate_on_the_host(lib):
     assert lib.awqmi_dev_fused_moe_block_rows(*big, 2 << 16) == 128
     assert lib.awqmi_dev_fused_moe_block_rows(*big, -1) == rows
     assert lib.awqmi_fused_moe_block_rows(*big) == rows
+
+
+def test_row_pitch_entry_points_validate_on_the_host(lib):
+    """awqmi_gemm_ld_f16 / awqmi_dequantize_ld_f16: the row pitch must cover a row and keep 16-byte
+    groups whole; everything else is checked as in the contiguous calls, before any launch."""
+    fake = 0x1000
+    assert lib.awqmi_gemm_ld_f16(fake, fake, 15, fake, fake, fake, 0, 0, 4, 1024, 128, 128, 0, 0) == 7   # pitch < N / 8
+    assert lib.awqmi_gemm_ld_f16(fake, fake, 18, fake, fake, fake, 0, 0, 4, 1024, 128, 128, 0, 0) == 7   # not % 4
+    assert lib.awqmi_gemm_ld_f16(fake, 0, 48, fake, fake, fake, 0, 0, 4, 1024, 128, 128, 0, 0) == 6
+    assert lib.awqmi_gemm_ld_f16(fake, fake, 48, fake, fake, fake, 0, 0, 4, 1000, 128, 128, 0, 0) == 1
+    assert lib.awqmi_dequantize_ld_f16(fake, 12, fake, fake, fake, 128, 128, 128, 0) == 7
+    assert lib.awqmi_dequantize_ld_f16(fake, 48, fake, fake, 0, 128, 128, 128, 0) == 6
+
+
+def test_pad_qweight_rows_and_the_method_hook(sba):
+    """A packed row that is a multiple of 1 KiB gets one 128-byte line of pitch more (same shape,
+    same values, a view of a wider buffer); any other row length is left alone.
+    AWQLinearMethod.process_weights_after_loading applies it and keeps qzeros / scales contiguous."""
+    import importlib
+    ops = importlib.import_module(sba.__name__ + ".ops")
+    g = torch.Generator().manual_seed(0)
+    q = torch.randint(-2**31, 2**31 - 1, (64, 256), dtype=torch.int32, generator=g)       # 1 KiB rows
+    p = ops.pad_qweight_rows(q)
+    assert tuple(p.shape) == (64, 256) and p.stride() == (288, 1) and torch.equal(p, q)
+    assert not p.is_contiguous() and p.data_ptr() != q.data_ptr()
+    q2 = torch.randint(-2**31, 2**31 - 1, (64, 160), dtype=torch.int32, generator=g)      # 640-byte rows
+    assert ops.pad_qweight_rows(q2) is q2
+    assert ops.pad_qweight_rows(p) is p                                                     # already padded
+    m = sba.AWQLinearMethod(sba.AWQConfig(4, 128, True))
+    layer = torch.nn.Module()
+    m.create_weights(layer, 256, [2048], 256, 2048, torch.float16)
+    layer.qweight.data.copy_(torch.randint(-2**31, 2**31 - 1, (256, 256), dtype=torch.int32, generator=g))
+    want = layer.qweight.data.clone()
+    m.process_weights_after_loading(layer)
+    assert layer.qweight.stride() == (288, 1) and torch.equal(layer.qweight.data, want)
+    assert layer.qzeros.is_contiguous() and layer.scales.is_contiguous()
+    assert sorted(n for n, _ in layer.named_parameters()) == ["qweight", "qzeros", "scales"]
 
 
 def test_fused_moe_workspace_covers_every_intermediate(lib):
@@ -497,6 +534,7 @@ def test_awq_gemm_takes_vllm_split_k_iters_as_a_hint(sba, monkeypatch):
 
     monkeypatch.setattr(libmod, "load", lambda: FakeLib())
     monkeypatch.setattr(ops, "_need", lambda *a, **k: None)
+    monkeypatch.setattr(ops, "_need_qweight", lambda t: t.shape[1])
     monkeypatch.setattr(ops, "_stream_ptr", lambda dev: 0)
     monkeypatch.setattr(ops, "get_workspace", lambda dev, n, s=None: torch.zeros(n, dtype=torch.uint8))
     monkeypatch.setattr(ops, "_gemm_ws_bytes", {})
