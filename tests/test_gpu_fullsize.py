@@ -127,3 +127,22 @@ def test_activations_beyond_4gib_run_as_row_slabs(sba, gpu):
         err = _rel(y[r0:r0 + 256], ref)
         print(f"[slabs] rows {r0}..{r0 + 255} rel_fro={err:.2e}", flush=True)
         assert err <= TOL
+
+
+@pytest.mark.parametrize("name,K,N", [("qkv_proj", 8192, 10240), ("o_proj", 8192, 8192), ("down_proj", 29568, 8192),
+                                      ("llama-70b gate_up", 8192, 57344)])
+def test_full_size_layers_in_the_methods_row_pitch(sba, gpu, name, K, N):
+    """Layers whose packed rows are a multiple of 1 KiB, as AWQLinearMethod holds them after
+    loading (rows one 128-byte line further apart): decode, 32-row and prefill launches and
+    awq_dequantize give the bits of the contiguous tensor."""
+    import importlib
+    ops = importlib.import_module(sba.__name__ + ".ops")
+    qw, sc, qz, g = _weights(K, N, gpu, 5)
+    qwp = ops.pad_qweight_rows(qw)
+    assert qwp.stride() == (N // 8 + 32, 1) and tuple(qwp.shape) == tuple(qw.shape)
+    for M in (1, 16, 32, 300):
+        x = torch.randn((M, K), device=gpu, generator=g).half()
+        y0 = sba.awq_gemm(x, qw, sc, qz, 0)
+        y1 = sba.awq_gemm(x, qwp, sc, qz, 0)
+        assert torch.equal(y0.view(torch.int16), y1.view(torch.int16)), (name, M)
+    assert torch.equal(sba.awq_dequantize(qw, sc, qz).view(torch.int16), sba.awq_dequantize(qwp, sc, qz).view(torch.int16))
