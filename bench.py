@@ -88,8 +88,8 @@ def main():
     ap.add_argument("--rows", choices=("contiguous", "method"), default="contiguous",
                     help="layout of the dense layers' qweight: contiguous as in the checkpoint (what the ops "
                          "awq_gemm / awq_dequantize are handed by vLLM's own method), or as this package's "
-                         "AWQLinearMethod.process_weights_after_loading holds it (rows that are a multiple of "
-                         "1 KiB get one 128-byte line of pitch more); the other layout's sweep is timed beside it")
+                         "AWQLinearMethod.process_weights_after_loading holds it (rows of N >= 8192 that are a "
+                         "multiple of 512 bytes get one 128-byte line of pitch more); the other layout's sweep is timed beside it")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--decoder", action="store_true", help=argparse.SUPPRESS)   # kept for old command lines
@@ -335,8 +335,8 @@ def main():
                                "16 awq_gemm launches per step, 4 rotating weight copies per layer",
                    "launch": args.launch, "split_k": args.split_k, "bytes_per_step": step_bytes,
                    "qweight_rows": ("as AWQLinearMethod.process_weights_after_loading holds them: int32 [K, N/8] "
-                                    "with the rows of qkv / o / down (multiples of 1 KiB) one 128-byte line further "
-                                    "apart, values and shapes unchanged, pad never read"
+                                    "with the rows of qkv / o / down (multiples of 512 bytes, 32 lines or more) one 128-byte "
+                                    "line further apart, values and shapes unchanged, pad never read"
                                     if args.rows == "method" else "contiguous, as in the checkpoint")},
         "other_qweight_rows": other_rows,
         "peaks": {"hbm_GBps": HBM_PEAK_GBS, "hbm_source": "MI355X published HBM3E bandwidth, 8 TB/s",

@@ -71,12 +71,14 @@ ROW_PAD_WORDS = 32      # one 128-byte line
 
 def pad_qweight_rows(qweight: torch.Tensor) -> torch.Tensor:
     """The same [K, N / 8] qweight as a view of a buffer whose rows are one 128-byte line further
-    apart, when the packed row is a multiple of eight lines (1 KiB); any other qweight is returned
-    as it is.  Every wave of the skinny kernel reads one line per row: with rows a multiple of
-    1 KiB apart all its requests share address bits 7 - 9 and the launch streams 12 - 20 % slower
-    than with any other row pitch (measured on 8192 x N layers, N from 49152 to 65536)."""
+    apart, when the packed row is a multiple of four lines (512 bytes) and at least 32 lines long;
+    any other qweight is returned as it is.  Every wave of the skinny kernel reads one line per
+    row: with rows a multiple of 1 KiB apart all its requests share address bits 7 - 9 and the
+    launch streams 12 - 20 % slower than with any other row pitch (8192 x N layers, N from 49152 to
+    65536); a multiple of 512 bytes costs 5 - 10 % (228- and 116-line rows).  Rows of fewer than 32
+    lines (N < 8192) measured the same either way."""
     K, NW = qweight.shape
-    if NW % 256 != 0 or not qweight.is_contiguous():
+    if NW % 128 != 0 or NW < 1024 or not qweight.is_contiguous():
         return qweight
     buf = torch.empty((K, NW + ROW_PAD_WORDS), dtype=qweight.dtype, device=qweight.device)
     buf[:, NW:].zero_()

@@ -464,17 +464,17 @@ def test_qweight_pitch_is_validated(sba, gpu):
 
 
 def test_linear_method_pads_kib_rows_and_matches_contiguous(sba, gpu):
-    """A layer whose packed rows are 1 KiB: process_weights_after_loading re-pitches qweight, apply
-    gives the bits of awq_gemm on the contiguous tensor at decode and prefill sizes."""
+    """A layer whose packed rows are 32 lines: process_weights_after_loading re-pitches qweight,
+    apply gives the bits of awq_gemm on the contiguous tensor at decode and prefill sizes."""
     cfg = sba.AWQConfig(4, 128, True)
     m = sba.AWQLinearMethod(cfg)
     layer = torch.nn.Module()
-    m.create_weights(layer, 1024, [2048], 1024, 2048, torch.float16, device=gpu)
-    x, qw, s, qz = _np_case(300, 1024, 2048, 128, seed=77)
+    m.create_weights(layer, 512, [8192], 512, 8192, torch.float16, device=gpu)
+    x, qw, s, qz = _np_case(300, 512, 8192, 128, seed=77)
     layer.load_state_dict({"qweight": torch.from_numpy(qw), "qzeros": torch.from_numpy(qz),
                            "scales": torch.from_numpy(s)})
     m.process_weights_after_loading(layer)
-    assert layer.qweight.stride() == (288, 1)
+    assert layer.qweight.stride() == (1056, 1)
     xd, qwd, sd, qzd = _dev(gpu, x, qw, s, qz)
     for rows in (1, 16, 40, 300):
         y = m.apply(layer, xd[:rows].contiguous())

@@ -120,26 +120,30 @@ def test_row_pitch_entry_points_validate_on_the_host(lib):
 
 
 def test_pad_qweight_rows_and_the_method_hook(sba):
-    """A packed row that is a multiple of 1 KiB gets one 128-byte line of pitch more (same shape,
-    same values, a view of a wider buffer); any other row length is left alone.
-    AWQLinearMethod.process_weights_after_loading applies it and keeps qzeros / scales contiguous."""
+    """A packed row of 32 lines or more that is a multiple of 512 bytes gets one 128-byte line of
+    pitch more (same shape, same values, a view of a wider buffer); any other row length is left
+    alone.  AWQLinearMethod.process_weights_after_loading applies it and keeps qzeros / scales
+    contiguous."""
     import importlib
     ops = importlib.import_module(sba.__name__ + ".ops")
     g = torch.Generator().manual_seed(0)
-    q = torch.randint(-2**31, 2**31 - 1, (64, 256), dtype=torch.int32, generator=g)       # 1 KiB rows
+    q = torch.randint(-2**31, 2**31 - 1, (16, 1024), dtype=torch.int32, generator=g)      # 32 lines
     p = ops.pad_qweight_rows(q)
-    assert tuple(p.shape) == (64, 256) and p.stride() == (288, 1) and torch.equal(p, q)
+    assert tuple(p.shape) == (16, 1024) and p.stride() == (1056, 1) and torch.equal(p, q)
     assert not p.is_contiguous() and p.data_ptr() != q.data_ptr()
-    q2 = torch.randint(-2**31, 2**31 - 1, (64, 160), dtype=torch.int32, generator=g)      # 640-byte rows
-    assert ops.pad_qweight_rows(q2) is q2
+    q4 = torch.randint(-2**31, 2**31 - 1, (8, 1152), dtype=torch.int32, generator=g)      # 36 lines: multiple of 4
+    assert ops.pad_qweight_rows(q4).stride() == (1184, 1)
+    for shape in ((16, 1056), (16, 1120), (64, 256), (64, 640)):                           # 33 / 35 / 8 / 20 lines
+        t = torch.zeros(shape, dtype=torch.int32)
+        assert ops.pad_qweight_rows(t) is t
     assert ops.pad_qweight_rows(p) is p                                                     # already padded
     m = sba.AWQLinearMethod(sba.AWQConfig(4, 128, True))
     layer = torch.nn.Module()
-    m.create_weights(layer, 256, [2048], 256, 2048, torch.float16)
-    layer.qweight.data.copy_(torch.randint(-2**31, 2**31 - 1, (256, 256), dtype=torch.int32, generator=g))
+    m.create_weights(layer, 128, [8192], 128, 8192, torch.float16)
+    layer.qweight.data.copy_(torch.randint(-2**31, 2**31 - 1, (128, 1024), dtype=torch.int32, generator=g))
     want = layer.qweight.data.clone()
     m.process_weights_after_loading(layer)
-    assert layer.qweight.stride() == (288, 1) and torch.equal(layer.qweight.data, want)
+    assert layer.qweight.stride() == (1056, 1) and torch.equal(layer.qweight.data, want)
     assert layer.qzeros.is_contiguous() and layer.scales.is_contiguous()
     assert sorted(n for n, _ in layer.named_parameters()) == ["qweight", "qzeros", "scales"]
 
