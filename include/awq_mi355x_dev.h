@@ -26,6 +26,9 @@
  *   1 << 23  dense skinny launches never share left-over chunks step by step
  *   1 << 24  the one-call MoE block always routes in a launch of its own (blocks of at most four
  *            tokens otherwise fold the routing into the first expert GEMM)
+ *   1 << 25  awq_gemm never takes the dequantise-once form (many-row calls run the fused kernel)
+ *   1 << 26  awq_gemm takes the dequantise-once form from 257 rows on, when the workspace holds
+ *            awqmi_dev_gemm_dense_workspace_bytes()
  * The workspace must be large enough for the form that is forced: the sizes the public queries
  * return cover every variant except a forced MFMA tile size, which silently runs without its K
  * split when the workspace is too small for it.
@@ -42,6 +45,20 @@ extern "C" {
 int awqmi_dev_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
                        const int32_t* qzeros, void* y_f16, void* workspace, size_t workspace_bytes,
                        int M, int K, int N, int group, int split_k, void* stream, int variant);
+
+/* Kernel family the last awqmi_gemm_* call on the calling thread launched. */
+enum {
+  AWQMI_FORM_NONE = 0,
+  AWQMI_FORM_SKINNY = 1,  /* awq_gemv_kernel: up to 32 rows per pass */
+  AWQMI_FORM_FUSED = 2,   /* awq_gemm_mfma_kernel: weights dequantised per tile in LDS */
+  AWQMI_FORM_DENSE = 3,   /* awq_dequant_panel_kernel + awq_gemm_dense_kernel */
+  AWQMI_FORM_GENERIC = 4  /* any-shape fallback */
+};
+int awqmi_dev_last_gemm_form(void);
+
+/* Workspace bytes with which a call of this shape can take the dequantise-once form (counters,
+ * K-split partial tiles, fp16 panel); 0 when the shape cannot (K % 64 != 0). */
+size_t awqmi_dev_gemm_dense_workspace_bytes(int M, int K, int N);
 
 int awqmi_dev_moe_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
                            const int32_t* qzeros, void* y_f16, const int32_t* sorted_token_ids,

@@ -53,6 +53,10 @@ for _name in ("awqmi_gemm_f16", "awqmi_moe_gemm_f16", "awqmi_fused_moe_routed_f1
     _res, _args = SIGNATURES[_name]
     SIGNATURES[_name.replace("awqmi_", "awqmi_dev_", 1)] = (_res, [*_args, c_int])
 
+SIGNATURES["awqmi_dev_last_gemm_form"] = (c_int, [])
+SIGNATURES["awqmi_dev_gemm_dense_workspace_bytes"] = (c_size_t, [c_int, c_int, c_int])
+FORM_SKINNY, FORM_FUSED, FORM_DENSE, FORM_GENERIC = 1, 2, 3, 4   # awqmi_dev_last_gemm_form()
+
 _lib = None
 
 

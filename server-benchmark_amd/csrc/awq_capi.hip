@@ -13,6 +13,7 @@
 #include "../../include/awq_mi355x.h"
 #include "../../include/awq_mi355x_dev.h"
 #include "awq_dequant.hpp"
+#include "awq_gemm_dense.hpp"
 #include "awq_gemm_mfma.hpp"
 #include "awq_gemv.hpp"
 #include "awq_moe.hpp"
@@ -29,6 +30,8 @@ static __device__ __align__(256) unsigned char scratch[AWQMI_STATIC_SCRATCH_BYTE
 namespace {
 
 thread_local int t_last_hip_error = 0;
+// which kernel family the last awqmi_gemm_* call on this thread launched (awqmi_dev_last_gemm_form)
+thread_local int t_last_gemm_form = 0;
 
 // Launch-rule variant of the call in progress on this thread: -1 (every default) for the whole
 // public C ABI; the awqmi_dev_* entry points set it for the duration of their own call only, so
@@ -58,6 +61,8 @@ enum : int {
   VAR_MFMA_ROWS_SHIFT = 20,   // bits 20..22 = v: MFMA tiles of 64 v rows (v = 1..4) whatever M is
   VAR_NO_TAIL_STEP = 1 << 23, // dense skinny launches never share left-over chunks step by step
   VAR_NO_FOLDED_ROUTE = 1 << 24, // the one-call MoE block always routes in a launch of its own
+  VAR_NO_DENSE = 1 << 25,        // awq_gemm never takes the dequantise-once form
+  VAR_DENSE = 1 << 26,           // awq_gemm takes the dequantise-once form from 257 rows on (workspace permitting)
 };
 inline bool variant_on(int bit) {
   return t_variant >= 0 && (t_variant & bit);
@@ -215,6 +220,22 @@ MfmaPlan plan_mfma(int M, int K, int N, int bm) {
   pl.sk_split = c;
   pl.part_bytes = (size_t)rem * c * PF_SK_SLOT_FLOATS * sizeof(float);
   return pl;
+}
+
+// Dequantise-once form (awq_gemm_dense.hpp): the weights go through awq_dequant_panel_kernel into
+// an fp16 panel in the workspace, then awq_gemm_dense_kernel.  The panel pass costs the time of
+// about 2900 rows' worth of what the dense kernel saves per row over the fused one (sustained
+// load, 72B layer shapes: 8192 rows 4 - 8 % faster, 2048 rows 2 - 5 % slower), so it is taken
+// from 4096 rows on.  K % 64 == 0 and G % 8 == 0 (both implied by the MFMA path's conditions).
+constexpr int DENSE_MIN_ROWS = 4096;
+inline bool dense_rows(int M) {
+  if (variant_on(VAR_NO_DENSE)) return false;
+  if (variant_on(VAR_DENSE)) return M > 256;
+  return M >= DENSE_MIN_ROWS;
+}
+// workspace of the dequantise-once form: counters, K-split partial tiles, then the panel
+inline size_t dense_panel_offset(size_t part_bytes) {
+  return (AWQMI_WS_COUNTER_BYTES + part_bytes + 1023) / 1024 * 1024;
 }
 
 // Rows of the MFMA tile (64, 128, 192 or 256) for one launch.  Smaller tiles pad less and give
@@ -439,6 +460,14 @@ size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
       // the tile rows the call will pick (a forced size that needs more falls back to no K split)
       mfma = plan_mfma(slab, K, N, mfma_pick_rows(slab, K, N)).part_bytes;
       if (M % slab) mfma = std::max(mfma, plan_mfma(M % slab, K, N, mfma_pick_rows(M % slab, K, N)).part_bytes);
+      // the dequantise-once form of many-row calls: 256-row tiles, and the fp16 panel behind the
+      // partial tiles (a call with a smaller workspace runs the fused kernel instead)
+      if (M >= DENSE_MIN_ROWS) {
+        size_t part = plan_mfma(slab, K, N, 256).part_bytes;
+        if (M % slab) part = std::max(part, plan_mfma(M % slab, K, N, 256).part_bytes);
+        const size_t dense = dense_panel_offset(part) + dg_panel_bytes(K, N) - AWQMI_WS_COUNTER_BYTES;
+        mfma = std::max(mfma, dense);
+      }
     }
   }
   if (M <= SKINNY_MAX_M) {
@@ -497,6 +526,7 @@ int awqmi_gemm_ld_f16(const void* x, const int32_t* qweight, int ldw, const void
       if (workspace_bytes < AWQMI_WS_COUNTER_BYTES + gemv_partial_bytes(N, split, 1, M > 16 ? 32 : 16))
         return AWQMI_WORKSPACE_TOO_SMALL;
     }
+    t_last_gemm_form = AWQMI_FORM_SKINNY;
     GemvParams p{};
     p.qw = qw; p.sc = sc; p.qz = qz;
     p.cnt = reinterpret_cast<int*>(workspace);
@@ -530,6 +560,41 @@ int awqmi_gemm_ld_f16(const void* x, const int32_t* qweight, int ldw, const void
   if (mfma_ok) {
     if (const int rc = ensure_kernel_attributes()) return rc;
     const int slab = mfma_slab_rows(M, K);
+    // many rows: dequantise once into the workspace, then the dense kernel (same bits as the fused
+    // kernel with 256-row tiles); needs the workspace to hold the panel
+    if (dense_rows(M) && workspace && aligned16(workspace)) {
+      size_t part = plan_mfma(slab < M ? slab : M, K, N, 256).part_bytes;
+      if (M % slab) part = std::max(part, plan_mfma(M % slab, K, N, 256).part_bytes);
+      const size_t panel_off = dense_panel_offset(part);
+      if (workspace_bytes >= panel_off + dg_panel_bytes(K, N)) {
+        t_last_gemm_form = AWQMI_FORM_DENSE;
+        unsigned char* const panel = static_cast<unsigned char*>(workspace) + panel_off;
+        const int nt = (N + 255) / 256;
+        hipLaunchKernelGGL(awq_dequant_panel_kernel, dim3(nt, K / 64), dim3(256), 0, st, qw, sc, qz, panel, K, N, NW, G,
+                           ldw);
+        for (int r0 = 0; r0 < M; r0 += slab) {
+          const int Ms = M - r0 < slab ? M - r0 : slab;
+          const MfmaPlan pl = plan_mfma(Ms, K, N, 256);
+          DenseGemmParams d{};
+          d.x = xx + (size_t)r0 * K; d.panel = panel; d.y = yy + (size_t)r0 * N;
+          d.M = Ms; d.K = K; d.N = N;
+          d.mt = (Ms + 255) / 256; d.nt = nt;
+          d.dp_tiles = pl.dp_tiles; d.sk_tiles = pl.sk_tiles; d.sk_split = pl.sk_split;
+          d.per_xcd = (pl.dp_tiles + 7) / 8;
+          d.sk_part = reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES);
+          hipLaunchKernelGGL((awq_gemm_dense_kernel<4>), dim3(d.per_xcd * 8 + d.sk_tiles * d.sk_split), dim3(256), 0, st,
+                             d);
+          if (d.sk_tiles > 0) {
+            MfmaGemmParams r{};
+            r.y = d.y; r.M = Ms; r.N = N; r.mt = d.mt; r.nt = nt;
+            r.dp_tiles = d.dp_tiles; r.sk_tiles = d.sk_tiles; r.sk_split = d.sk_split; r.sk_part = d.sk_part;
+            hipLaunchKernelGGL((awq_gemm_mfma_reduce_kernel<4, 4>), dim3(d.sk_tiles * 16), dim3(256), 0, st, r);
+          }
+        }
+        return launch_status();
+      }
+    }
+    t_last_gemm_form = AWQMI_FORM_FUSED;
     for (int r0 = 0; r0 < M; r0 += slab) {
       const int Ms = M - r0 < slab ? M - r0 : slab;
       MfmaGemmParams p{};
@@ -579,6 +644,7 @@ int awqmi_gemm_ld_f16(const void* x, const int32_t* qweight, int ldw, const void
 
   // any other shape: one thread per packed word and row; the row index is the grid's second
   // dimension (at most 65535), so more rows run as consecutive slabs
+  t_last_gemm_form = AWQMI_FORM_GENERIC;
   for (int r0 = 0; r0 < M; r0 += 32768) {
     const int Ms = M - r0 < 32768 ? M - r0 : 32768;
     hipLaunchKernelGGL(awq_gemm_generic_kernel, dim3((NW + 255) / 256, Ms), dim3(256), 0, st,
@@ -1117,6 +1183,17 @@ int awqmi_dev_gemm_f16(const void* x, const int32_t* qweight, const void* scales
                        int split_k, void* stream, int variant) {
   VariantScope scope(variant);
   return awqmi_gemm_f16(x, qweight, scales, qzeros, y, workspace, workspace_bytes, M, K, N, group, split_k, stream);
+}
+
+int awqmi_dev_last_gemm_form(void) { return t_last_gemm_form; }
+
+size_t awqmi_dev_gemm_dense_workspace_bytes(int M, int K, int N) {
+  if (M <= 0 || K <= 0 || N <= 0 || K % 64 != 0) return 0;
+  const int slab = mfma_slab_rows(M, K);
+  if (slab <= 0) return 0;
+  size_t part = plan_mfma(slab, K, N, 256).part_bytes;
+  if (M % slab) part = std::max(part, plan_mfma(M % slab, K, N, 256).part_bytes);
+  return dense_panel_offset(part) + dg_panel_bytes(K, N);
 }
 
 int awqmi_dev_moe_gemm_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,

@@ -19,6 +19,8 @@ _WS_COUNTER_BYTES = 65536
 _workspaces: dict = {}
 _retired: list = []      # outgrown workspaces, kept because captured graphs may still point at them
 _gemm_ws_bytes: dict = {}  # (M, K, N, split) -> awqmi_gemm_workspace_bytes, asked once per shape
+DEV_VARIANT_NO_DENSE = 1 << 25   # development variant bits of awq_gemm (include/awq_mi355x_dev.h)
+DEV_VARIANT_DENSE = 1 << 26
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -174,6 +176,9 @@ def awq_gemm(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
     nbytes = _gemm_ws_bytes.get(shape_key)
     if nbytes is None:
         nbytes = _gemm_ws_bytes[shape_key] = lib.awqmi_gemm_workspace_bytes(M, K, N, split)
+    if _dev_variant is not None and _dev_variant >= 0 and (_dev_variant & DEV_VARIANT_DENSE):
+        # the dequantise-once form forced below the row count at which the workspace query counts on it
+        nbytes = max(nbytes, lib.awqmi_dev_gemm_dense_workspace_bytes(M, K, N))
     stream = _stream_ptr(input.device)
     ws = get_workspace(input.device, nbytes, stream)
     args = (input.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(), out.data_ptr(),

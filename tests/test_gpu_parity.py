@@ -346,6 +346,56 @@ def test_gemm_prefill_partial_rounds(sba, gpu, M, K, N):
     assert np.array_equal(y1.view(np.uint16), y2.view(np.uint16))      # deterministic
 
 
+@pytest.mark.parametrize("M,K,N,G", [(300, 1024, 520, 128), (512, 2048, 1024, 128), (257, 192, 264, 32),
+                                     (700, 256, 264, 64), (1024, 512, 1280, 128), (2048, 512, 5120, 128),
+                                     (768, 1536, 8192 + 256, 128), (1500, 384, 2056, -1), (4100, 320, 776, 64)])
+def test_gemm_dequantise_once_form(sba, gpu, M, K, N, G):
+    """The many-row form (weights dequantised once into a panel in the workspace, then the dense
+    kernel fed by direct-to-LDS loads), forced through the development entry point at small
+    shapes: ragged rows and columns, stage counts that are not a multiple of the ring length,
+    a K split of a sparse last round, groups of 32 / 64 / 128 / K.  Checked against the oracle, and
+    bit for bit against the fused kernel with 256-row tiles (same k-step order, same split)."""
+    from server_benchmark_amd import _lib, ops
+    lib = _lib.load()
+    g = K if G <= 0 else G
+    x, qw, s, qz = _np_case(M, K, N, G, seed=M + 3 * N)
+    y_dense = _check_gemm(sba, gpu, x, qw, s, qz, g, 0, tag="dense form", variant=ops.DEV_VARIANT_DENSE)
+    assert lib.awqmi_dev_last_gemm_form() == _lib.FORM_DENSE
+    y_fused = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), 0, _dev_variant=ops.DEV_VARIANT_NO_DENSE | (4 << 20)).cpu().numpy()
+    assert lib.awqmi_dev_last_gemm_form() == _lib.FORM_FUSED
+    assert np.array_equal(y_dense.view(np.uint16), y_fused.view(np.uint16))
+    y_again = sba.awq_gemm(*_dev(gpu, x, qw, s, qz), 0, _dev_variant=ops.DEV_VARIANT_DENSE).cpu().numpy()
+    assert np.array_equal(y_dense.view(np.uint16), y_again.view(np.uint16))
+
+
+def test_gemm_dequantise_once_default_rule_and_small_workspace(sba, gpu):
+    """From 4096 rows on the public entry point takes the dequantise-once form when the workspace
+    holds the panel (a row-padded qweight included) and the fused kernel when it does not; both
+    return the same bits."""
+    from server_benchmark_amd import _lib, ops
+    lib = _lib.load()
+    M, K, N, G = 4096, 256, 1024 * 8, 128
+    x, qw, s, qz = _np_case(M, K, N, G, seed=11)
+    xd, qwd, sd, qzd = _dev(gpu, x, qw, s, qz)
+    y = sba.awq_gemm(xd, qwd, sd, qzd, 0)
+    assert lib.awqmi_dev_last_gemm_form() == _lib.FORM_DENSE
+    padded = ops.pad_qweight_rows(qwd)
+    assert not padded.is_contiguous()
+    y_pad = sba.awq_gemm(xd, padded, sd, qzd, 0)
+    assert lib.awqmi_dev_last_gemm_form() == _lib.FORM_DENSE
+    assert torch.equal(y, y_pad)
+    # a workspace without room for the panel: the same call runs the fused kernel
+    small = torch.zeros(lib.awqmi_gemm_workspace_bytes(2048, K, N, 0), dtype=torch.uint8, device=gpu)
+    y_small = torch.empty_like(y)
+    st = lib.awqmi_gemm_f16(xd.data_ptr(), qwd.data_ptr(), sd.data_ptr(), qzd.data_ptr(), y_small.data_ptr(),
+                            small.data_ptr(), small.numel(), M, K, N, G, 0, torch.cuda.current_stream().cuda_stream)
+    assert st == 0 and lib.awqmi_dev_last_gemm_form() == _lib.FORM_FUSED
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_small)
+    ref = awq_ref.gemm_wide(x[:64], qw, s, qz, G)
+    assert awq_ref.rel_frobenius(y[:64].cpu().numpy(), ref) <= TOL
+
+
 @pytest.mark.parametrize("M,K,N,G", [(3, 96, 40, 32), (20, 100, 16, 50), (2, 24, 8, 8)])
 def test_gemm_generic_fallback(sba, gpu, M, K, N, G):
     x, qw, s, qz = _np_case(M, K, N, G, seed=5)

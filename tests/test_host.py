@@ -204,7 +204,13 @@ def test_workspace_and_split_k_queries(lib):
         assert need >= 65536
         if s > 1:
             assert need >= 65536 + s * 16 * N * 4
-    assert lib.awqmi_gemm_workspace_bytes(8192, 8192, 8192, 0) == 65536     # whole rounds: no partials
+    assert lib.awqmi_gemm_workspace_bytes(2048, 8192, 8192, 0) == 65536     # whole rounds: no partials
+    # from 4096 rows on: room for the fp16 panel of the dequantise-once form (K * N * 2 bytes for
+    # whole 256-column tiles) behind the counters
+    assert lib.awqmi_gemm_workspace_bytes(8192, 8192, 8192, 0) == 65536 + 8192 * 8192 * 2
+    assert lib.awqmi_gemm_workspace_bytes(4096, 8192, 8192 + 8, 0) >= 65536 + 8192 * (8192 + 256) * 2
+    assert lib.awqmi_dev_gemm_dense_workspace_bytes(8192, 8192, 8192) == 65536 + 8192 * 8192 * 2
+    assert lib.awqmi_dev_gemm_dense_workspace_bytes(300, 1000, 512) == 0    # K no multiple of 64
     assert lib.awqmi_gemm_workspace_bytes(512, 8192, 8192, 0) == 65536 + 64 * 4 * 256 * 256 * 4   # K split
     assert lib.awqmi_gemm_auto_split_k(512, 8192, 8192, 128) == 1
     assert lib.awqmi_gemm_workspace_bytes(32, 8192, 8192, 8) >= 65536 + 8 * 32 * 8192 * 4
