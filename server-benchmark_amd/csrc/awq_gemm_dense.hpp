@@ -8,24 +8,26 @@
 // both operands go from global memory straight into LDS (`buffer_load_dwordx4 ... lds`).
 //
 // Panel layout.  The panel is not [K, N]: it is the sequence of LDS images the GEMM wants.
-// Block (column tile c, k-stage t) of 16 KiB, at byte ((c * K / 32 + t) * 16384), holds the 256
-// columns of tile c for k = 32 t .. 32 t + 31 as [column][4 slots of 8 halves], slot l of
-// column j stored at physical slot l ^ ((j >> 2) & 3).  A k-stage of a column tile is one
-// contiguous 16 KiB run, so its fetch is 16 fully coalesced 1 KiB wave loads, and all k-stages
+// Block (column tile c, k-stage t) of 32 KiB, at byte ((c * K / 64 + t) * 32768), holds the 256
+// columns of tile c for k = 64 t .. 64 t + 63 as [column][8 slots of 8 halves], slot l of
+// column j stored at physical slot l ^ ((j >> 1) & 7).  A k-stage of a column tile is one
+// contiguous 32 KiB run, so its fetch is 32 fully coalesced 1 KiB wave loads, and all k-stages
 // of a column tile are consecutive in memory.  Columns past N hold zeros.
 //
-// LDS.  A ring of NST stages of 32 KiB (X tile 256 x 32, W tile 256 x 32, both [row][64 B] with
-// the slot swizzle above: 16 consecutive lanes of a fragment read -- rows i .. i + 15, one
-// logical slot -- touch 16 different 16-byte bank groups).  Stage t + NST is requested as soon
-// as every wave has left stage t, NST - 1 stage times before it is needed.  Every ring slot is an
-// LDS object of its own, so that the compiler's wait before reading a slot counts only the
-// loads issued after that slot's.
+// LDS.  Two stages of 64 KiB (X tile 256 x 64, W tile 256 x 64, both [row][128 B] with the slot
+// swizzle above: the 16 consecutive lanes of a fragment read -- rows i .. i + 15, one logical
+// slot -- touch 16 different 16-byte bank groups; an X row of a stage is one whole 128-byte
+// line).  Stage t + 2 is requested as soon as every wave has left stage t.  Each stage is an LDS
+// object of its own, so that the compiler's wait before reading one counts only the loads
+// issued after it.
 //
-// Workgroup tile 256 x 256, four waves 2 x 2, each 128 x 128 = 4 x 4 v_mfma_f32_32x32x16_f16
-// accumulators (the arrangement with the fewest LDS bytes per flop that fits the register
-// file).  Per stage a wave issues 32 MFMAs, 16 fragment reads, 8 direct-to-LDS loads and one
-// barrier.  The k-steps are accumulated in the same order as in the fused kernel, so for the
-// same K split both kernels return the same bits.
+// Workgroup tile 256 x 256, four waves 2 x 2, each 128 x 128 = 8 x 8 v_mfma_f32_16x16x32_f16
+// accumulators.  The 16 x 16 x 32 shape is the one that gives the most flops under the chip's
+// power limit: a bare loop of it holds 2.0 GHz with random operands where the 32 x 32 x 16 shape
+// holds 1.6 GHz (1.78 against 1.65 PFLOP/s sustained).  The weights are the A operand and the
+// activations the B operand, so that a lane's four accumulator values of a tile are four
+// consecutive output columns of one row (8-byte stores).  Per stage a wave issues 128 MFMAs,
+// 32 fragment reads, 16 direct-to-LDS loads and one barrier.
 #pragma once
 #include <type_traits>
 
@@ -34,12 +36,12 @@
 
 namespace awqmi {
 
-constexpr int DG_BK = 32;                           // k per stage
-constexpr int DG_ROW_BYTES = DG_BK * 2;             // 64 B per row and stage
-constexpr int DG_OP_BYTES = 256 * DG_ROW_BYTES;     // 16 KiB per operand and stage
+constexpr int DG_BK = 64;                           // k per stage
+constexpr int DG_ROW_BYTES = DG_BK * 2;             // 128 B per row and stage
+constexpr int DG_OP_BYTES = 256 * DG_ROW_BYTES;     // 32 KiB per operand and stage
 constexpr int DG_STAGE_BYTES = 2 * DG_OP_BYTES;     // X tile, then W tile
 
-__host__ __device__ constexpr int dg_swz(int row) { return (row >> 2) & 3; }
+__host__ __device__ constexpr int dg_swz(int row) { return (row >> 1) & 7; }
 
 // bytes of the panel of a [K, N] weight matrix (K % 64 == 0)
 __host__ __device__ constexpr size_t dg_panel_bytes(int K, int N) {
@@ -47,11 +49,11 @@ __host__ __device__ constexpr size_t dg_panel_bytes(int K, int N) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Dequantise into the panel.  One workgroup per (column tile, 64 rows of K): thread (kk, wcl)
-// takes rows 8 kk .. 8 kk + 7 of packed word column wcl of the tile, i.e. for each of its eight
-// logical columns one run of eight consecutive k = one 16-byte slot of the panel.  The 32 KiB
-// (two k-stages) are collected in LDS and leave as 16-byte stores in address order.
-// G % 8 == 0 (a thread's eight rows share a group).
+// Dequantise into the panel.  One workgroup per (column tile, k-stage): thread (kk, wcl) takes
+// rows 8 kk .. 8 kk + 7 of packed word column wcl of the tile, i.e. for each of its eight logical
+// columns one run of eight consecutive k = one 16-byte slot of the panel.  The 32 KiB are
+// collected in LDS and leave as 16-byte stores in address order.  G % 8 == 0 (a thread's eight
+// rows share a group).
 __global__ __launch_bounds__(256) void awq_dequant_panel_kernel(const uint32_t* __restrict__ qw,
                                                                 const half_t* __restrict__ sc,
                                                                 const uint32_t* __restrict__ qz,
@@ -59,7 +61,7 @@ __global__ __launch_bounds__(256) void awq_dequant_panel_kernel(const uint32_t* 
                                                                 int NW, int G, int ldw) {
   // staging layout: 16-byte unit (kk, column j) at kk * 4096 + (j >> 3) * 128 + (((j & 7) ^ ((j >> 4) & 7)) << 4):
   // the 32 lanes that store one column each (j = 8 wcl + c) spread over all bank groups
-  __shared__ __align__(16) unsigned char tile[2 * DG_OP_BYTES];
+  __shared__ __align__(16) unsigned char tile[DG_OP_BYTES];
   const int tid = threadIdx.x;
   const int nt_i = blockIdx.x, k64 = blockIdx.y;
   const int kk = tid >> 5, wcl = tid & 31;
@@ -105,12 +107,12 @@ __global__ __launch_bounds__(256) void awq_dequant_panel_kernel(const uint32_t* 
   byte_runs(std::integral_constant<int, 2>{});
   byte_runs(std::integral_constant<int, 3>{});
   __syncthreads();
-  unsigned char* dst = panel + ((size_t)nt_i * (size_t)(K / DG_BK) + 2 * (size_t)k64) * DG_OP_BYTES;
+  unsigned char* dst = panel + ((size_t)nt_i * (size_t)(K / DG_BK) + (size_t)k64) * DG_OP_BYTES;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int q = i * 256 + tid;                 // 16-byte unit of the two stage blocks, in address order
-    const int stage = q >> 10, row = (q >> 2) & 255, ps = q & 3;
-    const int skk = stage * 4 + (ps ^ dg_swz(row));
+    const int q = i * 256 + tid;                 // 16-byte unit of the stage block, in address order
+    const int row = q >> 3, ps = q & 7;
+    const int skk = ps ^ dg_swz(row);
     const int swc = row >> 3;
     const u4v v = *reinterpret_cast<const u4v*>(tile + skk * 4096 + swc * 128 + (((row & 7) ^ ((swc >> 1) & 7)) << 4));
     __builtin_nontemporal_store(v, reinterpret_cast<u4v*>(dst + (size_t)q * 16));
@@ -134,27 +136,31 @@ struct DenseGemmParams {
 // Wait until at most VM of this thread's loads are outstanding and its LDS reads have returned,
 // then the workgroup barrier.  Written as one asm statement with a memory clobber: no LDS access
 // moves across it, and the compiler's own fences, which would wait for every direct-to-LDS load
-// in flight (vmcnt(0)), stay out.
+// in flight whatever VM says, stay out.
 template <int VM>
 __device__ __forceinline__ void dg_wait_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(VM) : "memory");
 }
 
-template <int NST>
+// acc += A(16 x 32) * B(32 x 16) with the accumulator tile in place in the accumulation
+// registers.  As an asm statement the result is tied to its input, which keeps each of the 64
+// tiles in one register tuple for the whole loop (as a builtin the allocator gives some results
+// other registers and then permutes the tiles at the loop's back edge: 2.4 moves per MFMA).
+// A tile is touched once per 64 MFMAs, so no dependent-issue wait states are needed.
+__device__ __forceinline__ void dg_mfma(f4& c, const h8& a, const h8& b) {
+  asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
 __global__ __launch_bounds__(256, 1) void awq_gemm_dense_kernel(const DenseGemmParams p) {
-  static_assert(NST >= 3 && NST <= 5, "ring of three to five 32 KiB stages");
   typedef __attribute__((address_space(3))) void lds_void;
   __shared__ __align__(1024) unsigned char st0[DG_STAGE_BYTES];
   __shared__ __align__(1024) unsigned char st1[DG_STAGE_BYTES];
-  __shared__ __align__(1024) unsigned char st2[DG_STAGE_BYTES];
-  __shared__ __align__(1024) unsigned char st3[NST > 3 ? DG_STAGE_BYTES : 16];
-  __shared__ __align__(1024) unsigned char st4[NST > 4 ? DG_STAGE_BYTES : 16];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int id = blockIdx.x;
-  const int KT64 = p.K / 64;
-  int nid = 0, kb = 0, ke = 2 * KT64, part = -1;
+  const int KT = p.K / DG_BK;
+  int nid = 0, kb = 0, ke = KT, part = -1;
   if (id < 8 * p.per_xcd) {
     nid = (id & 7) * p.per_xcd + (id >> 3);
     if (nid >= p.dp_tiles) return;
@@ -162,8 +168,8 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_dense_kernel(const DenseGemmP
     const int j = id - 8 * p.per_xcd;
     nid = p.dp_tiles + j / p.sk_split;
     part = j % p.sk_split;
-    kb = 2 * (int)((long long)KT64 * part / p.sk_split);
-    ke = 2 * (int)((long long)KT64 * (part + 1) / p.sk_split);
+    kb = (int)((long long)KT * part / p.sk_split);
+    ke = (int)((long long)KT * (part + 1) / p.sk_split);
   }
   const int gsize = PF_GROUP_M * p.nt;
   const int first_m = (nid / gsize) * PF_GROUP_M;
@@ -174,183 +180,192 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_dense_kernel(const DenseGemmP
   const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
 
   const __amdgpu_buffer_rsrc_t rx = pf_rsrc(p.x, (size_t)p.M * p.K * 2);
-  const size_t col_tile_bytes = (size_t)(p.K / DG_BK) * DG_OP_BYTES;
+  const size_t col_tile_bytes = (size_t)KT * DG_OP_BYTES;
   const __amdgpu_buffer_rsrc_t rw = pf_rsrc(p.panel + (size_t)nt_i * col_tile_bytes, col_tile_bytes);
 
   // ---- global -> LDS roles ---------------------------------------------------------------
-  // X: instruction i of wave w fills rows 16 (4 i + w) .. + 15 of the stage (1 KiB); lane l
-  // lands in row + l / 4, physical slot l % 4, so it fetches logical slot (l % 4) ^ swz(row),
-  // and swz(row) = (l >> 4) & 3 for every i.  Rows past M re-read row M - 1 (never stored).
-  uint32_t x_voff[4];
+  // X: instruction i of wave w fills rows 8 (4 i + w) .. + 7 of the stage (1 KiB); lane l lands in
+  // row + l / 8, physical slot l % 8, so it fetches logical slot (l % 8) ^ swz(row), and
+  // swz(row) = (l >> 4) + 4 (w & 1) for every i.  Rows past M re-read row M - 1 (never stored).
+  uint32_t x_voff[8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = 16 * (4 * i + wave) + (lane >> 2);
+  for (int i = 0; i < 8; ++i) {
+    const int r = 8 * (4 * i + wave) + (lane >> 3);
     const int gr = min(m0 + r, p.M - 1);
-    x_voff[i] = (uint32_t)(((size_t)gr * p.K + 8 * ((lane & 3) ^ ((lane >> 4) & 3))) * 2);
+    x_voff[i] = (uint32_t)(((size_t)gr * p.K + 8 * ((lane & 7) ^ dg_swz(r))) * 2);
   }
   // W: the stage block is the LDS image; instruction i of wave w copies its KiB 4 i + w
   const uint32_t w_voff = (uint32_t)lane * 16u;
 
   // ---- LDS -> fragment roles -------------------------------------------------------------
-  // lane (fi = lane % 32, fh = lane / 32) reads row base + fi, logical slot 2 ks + fh
-  const int fi = lane & 31, fh = lane >> 5;
-  uint32_t fa_off[2], fb_off[2];
+  // lane (fi = lane % 16, fq = lane / 16) reads row base + fi, logical slot 4 ks + fq
+  const int fi = lane & 15, fq = lane >> 4;
+  uint32_t fx_off[2], fw_off[2];
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) {
-    const uint32_t o = (uint32_t)(fi * DG_ROW_BYTES + (((2 * ks + fh) ^ dg_swz(fi)) << 4));
-    fa_off[ks] = o + (uint32_t)(wm * DG_ROW_BYTES);
-    fb_off[ks] = o + (uint32_t)(DG_OP_BYTES + wn * DG_ROW_BYTES);
+    const uint32_t o = (uint32_t)(fi * DG_ROW_BYTES + (((4 * ks + fq) ^ dg_swz(fi)) << 4));
+    fx_off[ks] = o + (uint32_t)(wm * DG_ROW_BYTES);
+    fw_off[ks] = o + (uint32_t)(DG_OP_BYTES + wn * DG_ROW_BYTES);
   }
 
-  f16v acc[4][4];
+  // acc[in][im]: columns n0 + wn + 16 in + 4 (lane / 16) + 0..3 of row m0 + wm + 16 im + lane % 16
+  f4 acc[8][8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int j = 0; j < 8; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
 
   auto slot_ptr = [&](auto STAG) -> unsigned char* {
-    constexpr int S = decltype(STAG)::value;
-    if constexpr (S == 0) return st0;
-    else if constexpr (S == 1) return st1;
-    else if constexpr (S == 2) return st2;
-    else if constexpr (S == 3) return st3;
-    else return st4;
+    if constexpr (decltype(STAG)::value == 0) return st0;
+    else return st1;
   };
-  // request k-stage kt into ring slot S (stages past the end fetch the last one again: the
-  // number of loads in flight behind any stage stays the same to the end of the loop)
-  auto issue = [&](auto STAG, int kt) {
-    unsigned char* const st = slot_ptr(STAG);
-    const int ktc = min(kt, ke - 1);
+  h8 xf[2][8], wf[2][8];
+
+  // One k-step of 64 MFMAs out of fragment set FS, in sixteen groups of four (one weight
+  // fragment against four activation fragments).  Between the groups go the 16 fragment reads of
+  // the next k-step (k-step KSN of stage buffer SR, into the other fragment set) and, with DMA
+  // set, the 16 direct-to-LDS loads of k-stage `kt_load` into stage buffer SL.  The order is
+  // pinned as written: the MFMAs are asm statements, which the scheduler's instruction groups
+  // cannot name.
+  auto kstep = [&](auto FS, auto SR, auto KSN, auto DMA, auto SL, int kt_load) {
+    constexpr int fs = decltype(FS)::value, ksn = decltype(KSN)::value;
+    const unsigned char* const sr = slot_ptr(SR);
+    unsigned char* const sl = slot_ptr(SL);
+    const int ktc = min(kt_load, ke - 1);
     const uint32_t sx = (uint32_t)ktc * DG_ROW_BYTES;
     const uint32_t sw = (uint32_t)ktc * DG_OP_BYTES + (uint32_t)wave * 1024u;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void*)(st + (4 * i + wave) * 1024), 16, x_voff[i], sx, 0, 0);
+    for (int g = 0; g < 16; ++g) {
+      const int i = g >> 1, j0 = 4 * (g & 1);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void*)(st + DG_OP_BYTES + (4 * i + wave) * 1024), 16, w_voff,
-                                               sw + (uint32_t)i * 4096u, 0, 0);
-  };
-
-  h8 af[2][4], bf[2][4];
-  auto frags = [&](auto STAG, auto KS, auto FS) {
-    constexpr int ks = decltype(KS)::value, fs = decltype(FS)::value;
-    const unsigned char* const st = slot_ptr(STAG);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) af[fs][i] = *reinterpret_cast<const h8*>(st + 32 * i * DG_ROW_BYTES + fa_off[ks]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) bf[fs][j] = *reinterpret_cast<const h8*>(st + 32 * j * DG_ROW_BYTES + fb_off[ks]);
-  };
-  auto mfma_step = [&](auto FS) {
-    constexpr int fs = decltype(FS)::value;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[fs][i], bf[fs][j], acc[i][j], 0, 0, 0);
+      for (int j = j0; j < j0 + 4; ++j) dg_mfma(acc[i][j], wf[fs][i], xf[fs][j]);
+      __builtin_amdgcn_sched_barrier(0);
+      // fragment g of the next k-step: weights first (the next k-step starts with wf[0], xf[0..3])
+      const int f = g >> 1;
+      if (g & 1) xf[fs ^ 1][f] = *reinterpret_cast<const h8*>(sr + 16 * f * DG_ROW_BYTES + fx_off[ksn]);
+      else wf[fs ^ 1][f] = *reinterpret_cast<const h8*>(sr + 16 * f * DG_ROW_BYTES + fw_off[ksn]);
+      if constexpr (decltype(DMA)::value) {
+        if (g & 1)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void*)(sl + DG_OP_BYTES + (4 * f + wave) * 1024), 16, w_voff,
+                                                   sw + (uint32_t)f * 4096u, 0, 0);
+        else
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void*)(sl + (4 * f + wave) * 1024), 16, x_voff[f], sx, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
 
-  // One k-stage kt in ring slot S.  On entry fragment set 0 holds its first k-step.
+  // One k-stage kt in stage buffer S.  On entry fragment set 0 holds its first k-step.
   auto body = [&](auto STAG, int kt) {
     constexpr int S = decltype(STAG)::value;
-    using SN = std::integral_constant<int, (S + 1) % NST>;
+    using SN = std::integral_constant<int, S ^ 1>;
     // first k-step from registers while the second one's fragments are read
-    frags(STAG, I1{}, I1{});
-    mfma_step(I0{});
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    kstep(I0{}, STAG, I1{}, I0{}, STAG, 0);
     // stage kt + 1 has landed (own loads; the barrier extends that to every thread's) and this
     // wave's reads of stage kt have returned
-    dg_wait_and_barrier<(NST - 2) * 8>();
+    dg_wait_and_barrier<0>();
     __builtin_amdgcn_sched_barrier(0);
-    // slot S is free: request stage kt + NST into it; second k-step from registers while the
+    // buffer S is free: request stage kt + 2 into it; second k-step from registers while the
     // first fragments of stage kt + 1 are read
-    issue(STAG, kt + NST);
-    frags(SN{}, I0{}, I0{});
-    mfma_step(I1{});
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    kstep(I1{}, SN{}, I0{}, I1{}, STAG, kt + 2);
   };
 
-  // prologue: fill the ring
-  issue(std::integral_constant<int, 0>{}, kb);
-  issue(std::integral_constant<int, 1>{}, kb + 1);
-  issue(std::integral_constant<int, 2>{}, kb + 2);
-  if constexpr (NST > 3) issue(std::integral_constant<int, 3>{}, kb + 3);
-  if constexpr (NST > 4) issue(std::integral_constant<int, 4>{}, kb + 4);
-  dg_wait_and_barrier<(NST - 1) * 8>();
-  frags(I0{}, I0{}, I0{});
-  __builtin_amdgcn_sched_barrier(0);
-  int kt = kb;
-  for (int full = (ke - kb) / NST; full > 0; --full, kt += NST) {
-    body(std::integral_constant<int, 0>{}, kt);
-    body(std::integral_constant<int, 1>{}, kt + 1);
-    body(std::integral_constant<int, 2>{}, kt + 2);
-    if constexpr (NST > 3) body(std::integral_constant<int, 3>{}, kt + 3);
-    if constexpr (NST > 4) body(std::integral_constant<int, 4>{}, kt + 4);
-  }
-  // the stages left over when the count is not a multiple of the ring length
-  if (kt < ke) {
-    body(std::integral_constant<int, 0>{}, kt);
-    if (kt + 1 < ke) {
-      body(std::integral_constant<int, 1>{}, kt + 1);
-      if (kt + 2 < ke) {
-        body(std::integral_constant<int, 2>{}, kt + 2);
-        if constexpr (NST > 4) {
-          if (kt + 3 < ke) body(std::integral_constant<int, 3>{}, kt + 3);
-        }
+  // prologue: both stage buffers requested, the first one waited for
+  {
+    const uint32_t swv = (uint32_t)wave * 1024u;
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      unsigned char* const st = s2 ? st1 : st0;
+      const int ktc = min(kb + s2, ke - 1);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void*)(st + (4 * i + wave) * 1024), 16, x_voff[i],
+                                                 (uint32_t)ktc * DG_ROW_BYTES, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void*)(st + DG_OP_BYTES + (4 * i + wave) * 1024), 16, w_voff,
+                                                 (uint32_t)ktc * DG_OP_BYTES + swv + (uint32_t)i * 4096u, 0, 0);
       }
     }
   }
-  // no load may still be writing this workgroup's LDS when it is handed to the next one
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  dg_wait_and_barrier<16>();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    wf[0][i] = *reinterpret_cast<const h8*>(st0 + 16 * i * DG_ROW_BYTES + fw_off[0]);
+    xf[0][i] = *reinterpret_cast<const h8*>(st0 + 16 * i * DG_ROW_BYTES + fx_off[0]);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  int kt = kb;
+  for (int full = (ke - kb) / 2; full > 0; --full, kt += 2) {
+    body(I0{}, kt);
+    body(I1{}, kt + 1);
+  }
+  if (kt < ke) body(I0{}, kt);
+  // no load may still be writing this workgroup's LDS when it is handed to the next one; the
+  // last MFMAs have left the pipe before their results are read (they are asm statements, for
+  // which the compiler inserts no wait states)
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
 
-  // ---- split-K tiles: fp32 partial to the workspace (layout of awq_gemm_mfma_reduce_kernel<4, 4>)
+  // ---- split-K tiles: fp32 partial to the workspace, [accumulator tile][thread] groups of four
   if (part >= 0) {
     const int tl = nid - p.dp_tiles;
     float* mine = p.sk_part + ((size_t)tl * p.sk_split + part) * PF_SK_SLOT_FLOATS;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; r += 4) {
-          const int q = ((i * 4 + j) * 16 + r) >> 2;
-          const f4 v = {acc[i][j][r], acc[i][j][r + 1], acc[i][j][r + 2], acc[i][j][r + 3]};
-          *reinterpret_cast<f4*>(mine + ((size_t)q * 256 + tid) * 4) = v;
-        }
-    return;
+      for (int j = 0; j < 8; ++j) *reinterpret_cast<f4*>(mine + ((size_t)(i * 8 + j) * 256 + tid) * 4) = acc[i][j];
+    return;   // summed and written out by awq_gemm_dense_reduce_kernel, launched behind this kernel
   }
 
-  // D[i][j] of a 32x32 tile: j = lane % 32, i = 8 * (r / 4) + 4 * (lane / 32) + r % 4
-  const int col_l = lane & 31, row_l = 4 * (lane >> 5);
+  const int col_l = 4 * (lane >> 4), row_l = lane & 15;
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int j = 0; j < 8; ++j) {
+    const int row = m0 + wm + 16 * j + row_l;
+    if (row >= p.M) continue;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int col = n0 + wn + 32 * j + col_l;
+    for (int i = 0; i < 8; ++i) {
+      const int col = n0 + wn + 16 * i + col_l;      // N % 8 == 0: the four columns are all inside or all outside
       if (col >= p.N) continue;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm + 32 * i + 8 * (r >> 2) + row_l + (r & 3);
-        if (row < p.M) p.y[(size_t)row * p.N + col] = (half_t)acc[i][j][r];
-      }
+      const h4 v = {(half_t)acc[i][j][0], (half_t)acc[i][j][1], (half_t)acc[i][j][2], (half_t)acc[i][j][3]};
+      *reinterpret_cast<h4*>(p.y + (size_t)row * p.N + col) = v;
     }
+  }
+}
+
+// Sum of the split-K partial tiles of awq_gemm_dense_kernel, parts added in index order.  One
+// workgroup takes eight accumulator tiles (one i, all j) of one output tile.
+__global__ __launch_bounds__(256) void awq_gemm_dense_reduce_kernel(const DenseGemmParams p) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tl = blockIdx.x >> 3, i = blockIdx.x & 7;
+  const int nid = p.dp_tiles + tl;
+  const int gsize = PF_GROUP_M * p.nt;
+  const int first_m = (nid / gsize) * PF_GROUP_M;
+  const int gm = min(p.mt - first_m, PF_GROUP_M);
+  const int mt_i = first_m + (nid % gsize) % gm;
+  const int nt_i = (nid % gsize) / gm;
+  const int m0 = mt_i * 256, n0 = nt_i * 256;
+  const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
+  const float* tile_base = p.sk_part + (size_t)tl * p.sk_split * PF_SK_SLOT_FLOATS;
+  f4 v[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = f4{0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < p.sk_split; ++s) {
+    f4 t[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      t[j] = *reinterpret_cast<const f4*>(tile_base + (size_t)s * PF_SK_SLOT_FLOATS + ((size_t)(i * 8 + j) * 256 + tid) * 4);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] += t[j];
+  }
+  const int col = n0 + wn + 16 * i + 4 * (lane >> 4);
+  if (col >= p.N) return;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int row = m0 + wm + 16 * j + (lane & 15);
+    if (row >= p.M) continue;
+    const h4 o = {(half_t)v[j][0], (half_t)v[j][1], (half_t)v[j][2], (half_t)v[j][3]};
+    *reinterpret_cast<h4*>(p.y + (size_t)row * p.N + col) = o;
+  }
 }
 
 }  // namespace awqmi
