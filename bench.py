@@ -421,8 +421,8 @@ def main():
                                     "50 ms of the same launches untimed (sustained: the chip holds a lower clock under "
                                     "this load than in its first milliseconds); TFLOPs_burst = 3 - 6 launches after two "
                                     "warm-up launches; aggregate = total flops / total time over the 12 points",
-                          "kernels": "awq_gemm_mfma_kernel (fused) below 4096 rows; awq_dequant_panel_kernel + "
-                                     "awq_gemm_dense_kernel from 4096 rows on (the panel pass is inside the timed call)",
+                          "kernels": "awq_gemm_mfma_kernel (fused) below 2048 rows; awq_dequant_panel_kernel + "
+                                     "awq_gemm_dense_kernel from 2048 rows on (the panel pass is inside the timed call)",
                           "points": pts}
         log(f"[bench] prefill sweep aggregate {agg:.1f} TFLOP/s sustained ({agg / MFMA_FP16_PEAK_TFLOPS:.1%} of fp16 MFMA "
             f"peak), {agg_burst:.1f} burst")

@@ -223,11 +223,12 @@ MfmaPlan plan_mfma(int M, int K, int N, int bm) {
 }
 
 // Dequantise-once form (awq_gemm_dense.hpp): the weights go through awq_dequant_panel_kernel into
-// an fp16 panel in the workspace, then awq_gemm_dense_kernel.  The panel pass costs the time of
-// about 2900 rows' worth of what the dense kernel saves per row over the fused one (sustained
-// load, 72B layer shapes: 8192 rows 4 - 8 % faster, 2048 rows 2 - 5 % slower), so it is taken
-// from 4096 rows on.  K % 64 == 0 and G % 8 == 0 (both implied by the MFMA path's conditions).
-constexpr int DENSE_MIN_ROWS = 4096;
+// an fp16 panel in the workspace, then awq_gemm_dense_kernel.  Under sustained load on the 72B
+// layer shapes (fused kernel against panel pass + dense kernel, timed in turn): 512 rows 0.70,
+// 1024 rows 0.79 - 0.90, 2048 rows 1.01 - 1.03, 3072 rows 1.01 - 1.07, 4096 rows 1.08, 8192 rows
+// 1.11 - 1.16 of the fused kernel's rate; so it is taken from 2048 rows on.  K % 64 == 0 and
+// G % 8 == 0 (both implied by the MFMA path's conditions).
+constexpr int DENSE_MIN_ROWS = 2048;
 inline bool dense_rows(int M) {
   if (variant_on(VAR_NO_DENSE)) return false;
   if (variant_on(VAR_DENSE)) return M > 256;
@@ -582,14 +583,9 @@ int awqmi_gemm_ld_f16(const void* x, const int32_t* qweight, int ldw, const void
           d.dp_tiles = pl.dp_tiles; d.sk_tiles = pl.sk_tiles; d.sk_split = pl.sk_split;
           d.per_xcd = (pl.dp_tiles + 7) / 8;
           d.sk_part = reinterpret_cast<float*>(static_cast<char*>(workspace) + AWQMI_WS_COUNTER_BYTES);
-          hipLaunchKernelGGL((awq_gemm_dense_kernel<4>), dim3(d.per_xcd * 8 + d.sk_tiles * d.sk_split), dim3(256), 0, st,
-                             d);
-          if (d.sk_tiles > 0) {
-            MfmaGemmParams r{};
-            r.y = d.y; r.M = Ms; r.N = N; r.mt = d.mt; r.nt = nt;
-            r.dp_tiles = d.dp_tiles; r.sk_tiles = d.sk_tiles; r.sk_split = d.sk_split; r.sk_part = d.sk_part;
-            hipLaunchKernelGGL((awq_gemm_mfma_reduce_kernel<4, 4>), dim3(d.sk_tiles * 16), dim3(256), 0, st, r);
-          }
+          hipLaunchKernelGGL(awq_gemm_dense_kernel, dim3(d.per_xcd * 8 + d.sk_tiles * d.sk_split), dim3(256), 0, st, d);
+          if (d.sk_tiles > 0)
+            hipLaunchKernelGGL(awq_gemm_dense_reduce_kernel, dim3(d.sk_tiles * 8), dim3(256), 0, st, d);
         }
         return launch_status();
       }

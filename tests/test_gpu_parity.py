@@ -369,12 +369,12 @@ def test_gemm_dequantise_once_form(sba, gpu, M, K, N, G):
 
 
 def test_gemm_dequantise_once_default_rule_and_small_workspace(sba, gpu):
-    """From 4096 rows on the public entry point takes the dequantise-once form when the workspace
+    """From 2048 rows on the public entry point takes the dequantise-once form when the workspace
     holds the panel (a row-padded qweight included) and the fused kernel when it does not; both
     return the same bits."""
     from server_benchmark_amd import _lib, ops
     lib = _lib.load()
-    M, K, N, G = 4096, 256, 1024 * 8, 128
+    M, K, N, G = 2048, 256, 1024 * 8, 128
     x, qw, s, qz = _np_case(M, K, N, G, seed=11)
     xd, qwd, sd, qzd = _dev(gpu, x, qw, s, qz)
     y = sba.awq_gemm(xd, qwd, sd, qzd, 0)
@@ -385,7 +385,7 @@ def test_gemm_dequantise_once_default_rule_and_small_workspace(sba, gpu):
     assert lib.awqmi_dev_last_gemm_form() == _lib.FORM_DENSE
     assert torch.equal(y, y_pad)
     # a workspace without room for the panel: the same call runs the fused kernel
-    small = torch.zeros(lib.awqmi_gemm_workspace_bytes(2048, K, N, 0), dtype=torch.uint8, device=gpu)
+    small = torch.zeros(lib.awqmi_gemm_workspace_bytes(1024, K, N, 0), dtype=torch.uint8, device=gpu)
     y_small = torch.empty_like(y)
     st = lib.awqmi_gemm_f16(xd.data_ptr(), qwd.data_ptr(), sd.data_ptr(), qzd.data_ptr(), y_small.data_ptr(),
                             small.data_ptr(), small.numel(), M, K, N, G, 0, torch.cuda.current_stream().cuda_stream)

@@ -204,8 +204,8 @@ def test_workspace_and_split_k_queries(lib):
         assert need >= 65536
         if s > 1:
             assert need >= 65536 + s * 16 * N * 4
-    assert lib.awqmi_gemm_workspace_bytes(2048, 8192, 8192, 0) == 65536     # whole rounds: no partials
-    # from 4096 rows on: room for the fp16 panel of the dequantise-once form (K * N * 2 bytes for
+    assert lib.awqmi_gemm_workspace_bytes(1024, 8192, 16384, 0) == 65536    # whole rounds: no partials
+    # from 2048 rows on: room for the fp16 panel of the dequantise-once form (K * N * 2 bytes for
     # whole 256-column tiles) behind the counters
     assert lib.awqmi_gemm_workspace_bytes(8192, 8192, 8192, 0) == 65536 + 8192 * 8192 * 2
     assert lib.awqmi_gemm_workspace_bytes(4096, 8192, 8192 + 8, 0) >= 65536 + 8192 * (8192 + 256) * 2
