@@ -14,12 +14,15 @@
 // contiguous 32 KiB run, so its fetch is 32 fully coalesced 1 KiB wave loads, and all k-stages
 // of a column tile are consecutive in memory.  Columns past N hold zeros.
 //
-// LDS.  Two stages of 64 KiB (X tile 256 x 64, W tile 256 x 64, both [row][128 B] with the slot
-// swizzle above: the 16 consecutive lanes of a fragment read -- rows i .. i + 15, one logical
+// LDS.  Five tile buffers of 32 KiB -- all 160 KiB of a CU -- each [row][128 B] with the slot
+// swizzle above (the 16 consecutive lanes of a fragment read -- rows i .. i + 15, one logical
 // slot -- touch 16 different 16-byte bank groups; an X row of a stage is one whole 128-byte
-// line).  Stage t + 2 is requested as soon as every wave has left stage t.  Each stage is an LDS
-// object of its own, so that the compiler's wait before reading one counts only the loads
-// issued after it.
+// line).  A stage (64 k) is an X tile and a W tile; four buffers hold the stage being multiplied
+// and the next one, and the fifth lets the X tile of the stage after that be requested half a
+// stage early, so that the direct-to-LDS loads are spread evenly over the loop (X tiles while
+// the first k-step of a stage is multiplied, W tiles during the second) instead of running at
+// the load path's full rate for half of the time.  Each buffer is an LDS object of its own, so
+// that the compiler's wait before reading one counts only the loads issued after it.
 //
 // Workgroup tile 256 x 256, four waves 2 x 2, each 128 x 128 = 8 x 8 v_mfma_f32_16x16x32_f16
 // accumulators.  The 16 x 16 x 32 shape is the one that gives the most flops under the chip's
@@ -153,8 +156,13 @@ __device__ __forceinline__ void dg_mfma(f4& c, const h8& a, const h8& b) {
 
 __global__ __launch_bounds__(256, 1) void awq_gemm_dense_kernel(const DenseGemmParams p) {
   typedef __attribute__((address_space(3))) void lds_void;
-  __shared__ __align__(1024) unsigned char st0[DG_STAGE_BYTES];
-  __shared__ __align__(1024) unsigned char st1[DG_STAGE_BYTES];
+  // five tile buffers of 32 KiB, the whole LDS of a CU: stage t keeps its X tile in buffer
+  // 2 t mod 5 and its W tile in buffer (2 t + 1) mod 5
+  __shared__ __align__(1024) unsigned char tb0[DG_OP_BYTES];
+  __shared__ __align__(1024) unsigned char tb1[DG_OP_BYTES];
+  __shared__ __align__(1024) unsigned char tb2[DG_OP_BYTES];
+  __shared__ __align__(1024) unsigned char tb3[DG_OP_BYTES];
+  __shared__ __align__(1024) unsigned char tb4[DG_OP_BYTES];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -184,7 +192,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_dense_kernel(const DenseGemmP
   const __amdgpu_buffer_rsrc_t rw = pf_rsrc(p.panel + (size_t)nt_i * col_tile_bytes, col_tile_bytes);
 
   // ---- global -> LDS roles ---------------------------------------------------------------
-  // X: instruction i of wave w fills rows 8 (4 i + w) .. + 7 of the stage (1 KiB); lane l lands in
+  // X: instruction i of wave w fills rows 8 (4 i + w) .. + 7 of the tile (1 KiB); lane l lands in
   // row + l / 8, physical slot l % 8, so it fetches logical slot (l % 8) ^ swz(row), and
   // swz(row) = (l >> 4) + 4 (w & 1) for every i.  Rows past M re-read row M - 1 (never stored).
   uint32_t x_voff[8];
@@ -205,7 +213,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_dense_kernel(const DenseGemmP
   for (int ks = 0; ks < 2; ++ks) {
     const uint32_t o = (uint32_t)(fi * DG_ROW_BYTES + (((4 * ks + fq) ^ dg_swz(fi)) << 4));
     fx_off[ks] = o + (uint32_t)(wm * DG_ROW_BYTES);
-    fw_off[ks] = o + (uint32_t)(DG_OP_BYTES + wn * DG_ROW_BYTES);
+    fw_off[ks] = o + (uint32_t)(wn * DG_ROW_BYTES);
   }
 
   // acc[in][im]: columns n0 + wn + 16 in + 4 (lane / 16) + 0..3 of row m0 + wm + 16 im + lane % 16
@@ -215,41 +223,47 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_dense_kernel(const DenseGemmP
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
 
-  auto slot_ptr = [&](auto STAG) -> unsigned char* {
-    if constexpr (decltype(STAG)::value == 0) return st0;
-    else return st1;
+  auto buf = [&](auto BTAG) -> unsigned char* {
+    constexpr int B = decltype(BTAG)::value;
+    if constexpr (B == 0) return tb0;
+    else if constexpr (B == 1) return tb1;
+    else if constexpr (B == 2) return tb2;
+    else if constexpr (B == 3) return tb3;
+    else return tb4;
+  };
+  auto load_x = [&](unsigned char* dst, int kt, int i) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void*)(dst + (4 * i + wave) * 1024), 16, x_voff[i],
+                                             (uint32_t)min(kt, ke - 1) * DG_ROW_BYTES, 0, 0);
+  };
+  auto load_w = [&](unsigned char* dst, int kt, int i) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void*)(dst + (4 * i + wave) * 1024), 16, w_voff,
+                                             (uint32_t)min(kt, ke - 1) * DG_OP_BYTES + (uint32_t)(4 * i + wave) * 1024u, 0, 0);
   };
   h8 xf[2][8], wf[2][8];
 
-  // One k-step of 64 MFMAs out of fragment set FS, in sixteen groups of four (one weight
-  // fragment against four activation fragments).  Between the groups go the 16 fragment reads of
-  // the next k-step (k-step KSN of stage buffer SR, into the other fragment set) and, with DMA
-  // set, the 16 direct-to-LDS loads of k-stage `kt_load` into stage buffer SL.  The order is
+  // One k-step of 64 MFMAs out of fragment set FS, in 32 pairs (one weight fragment against two
+  // activation fragments).  Between the pairs go the 16 fragment reads of the next k-step (k-step
+  // KSN of tiles xr / wr, into the other fragment set) and eight direct-to-LDS loads: of the X
+  // tile (WLOAD = 0) or the W tile (WLOAD = 1) of k-stage kt_load into buffer dst.  The order is
   // pinned as written: the MFMAs are asm statements, which the scheduler's instruction groups
   // cannot name.
-  auto kstep = [&](auto FS, auto SR, auto KSN, auto DMA, auto SL, int kt_load) {
+  auto kstep = [&](auto FS, const unsigned char* xr, const unsigned char* wr, auto KSN, auto WLOAD, unsigned char* dst,
+                   int kt_load) {
     constexpr int fs = decltype(FS)::value, ksn = decltype(KSN)::value;
-    const unsigned char* const sr = slot_ptr(SR);
-    unsigned char* const sl = slot_ptr(SL);
-    const int ktc = min(kt_load, ke - 1);
-    const uint32_t sx = (uint32_t)ktc * DG_ROW_BYTES;
-    const uint32_t sw = (uint32_t)ktc * DG_OP_BYTES + (uint32_t)wave * 1024u;
 #pragma unroll
-    for (int g = 0; g < 16; ++g) {
-      const int i = g >> 1, j0 = 4 * (g & 1);
-#pragma unroll
-      for (int j = j0; j < j0 + 4; ++j) dg_mfma(acc[i][j], wf[fs][i], xf[fs][j]);
+    for (int h = 0; h < 32; ++h) {
+      const int i = h >> 2, j0 = 2 * (h & 3);
+      dg_mfma(acc[i][j0], wf[fs][i], xf[fs][j0]);
+      dg_mfma(acc[i][j0 + 1], wf[fs][i], xf[fs][j0 + 1]);
       __builtin_amdgcn_sched_barrier(0);
-      // fragment g of the next k-step: weights first (the next k-step starts with wf[0], xf[0..3])
-      const int f = g >> 1;
-      if (g & 1) xf[fs ^ 1][f] = *reinterpret_cast<const h8*>(sr + 16 * f * DG_ROW_BYTES + fx_off[ksn]);
-      else wf[fs ^ 1][f] = *reinterpret_cast<const h8*>(sr + 16 * f * DG_ROW_BYTES + fw_off[ksn]);
-      if constexpr (decltype(DMA)::value) {
-        if (g & 1)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void*)(sl + DG_OP_BYTES + (4 * f + wave) * 1024), 16, w_voff,
-                                                   sw + (uint32_t)f * 4096u, 0, 0);
-        else
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void*)(sl + (4 * f + wave) * 1024), 16, x_voff[f], sx, 0, 0);
+      // at most one memory instruction per pair of MFMAs (weights first: the next k-step starts
+      // with wf[0], xf[0..1])
+      const int f = h >> 2;
+      if ((h & 3) == 0) wf[fs ^ 1][f] = *reinterpret_cast<const h8*>(wr + 16 * f * DG_ROW_BYTES + fw_off[ksn]);
+      else if ((h & 3) == 2) xf[fs ^ 1][f] = *reinterpret_cast<const h8*>(xr + 16 * f * DG_ROW_BYTES + fx_off[ksn]);
+      else if ((h & 3) == 1) {
+        if constexpr (decltype(WLOAD)::value) load_w(dst, kt_load, f);
+        else load_x(dst, kt_load, f);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -257,50 +271,64 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_dense_kernel(const DenseGemmP
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
 
-  // One k-stage kt in stage buffer S.  On entry fragment set 0 holds its first k-step.
-  auto body = [&](auto STAG, int kt) {
-    constexpr int S = decltype(STAG)::value;
-    using SN = std::integral_constant<int, S ^ 1>;
-    // first k-step from registers while the second one's fragments are read
-    kstep(I0{}, STAG, I1{}, I0{}, STAG, 0);
-    // stage kt + 1 has landed (own loads; the barrier extends that to every thread's) and this
-    // wave's reads of stage kt have returned
-    dg_wait_and_barrier<0>();
+  // One k-stage kt, R = (kt - kb) mod 5.  On entry fragment set 0 holds its first k-step, its
+  // tiles and stage kt + 1's W tile are in LDS or on their way, and one buffer is free.
+  auto body = [&](auto RTAG, int kt) {
+    constexpr int R = decltype(RTAG)::value;
+    unsigned char* const xb = buf(std::integral_constant<int, (2 * R) % 5>{});
+    unsigned char* const wb = buf(std::integral_constant<int, (2 * R + 1) % 5>{});
+    unsigned char* const xn = buf(std::integral_constant<int, (2 * R + 2) % 5>{});
+    unsigned char* const wn_ = buf(std::integral_constant<int, (2 * R + 3) % 5>{});
+    unsigned char* const spare = buf(std::integral_constant<int, (2 * R + 4) % 5>{});
+    // first k-step from registers while the second one's fragments are read and the X tile of
+    // stage kt + 2 is requested into the free buffer
+    kstep(I0{}, xb, wb, I1{}, I0{}, spare, kt + 2);
+    // stage kt + 1 has landed -- everything but the eight loads just issued (own loads; the
+    // barrier extends that to every thread's) -- and this wave's reads of stage kt have returned
+    dg_wait_and_barrier<8>();
     __builtin_amdgcn_sched_barrier(0);
-    // buffer S is free: request stage kt + 2 into it; second k-step from registers while the
-    // first fragments of stage kt + 1 are read
-    kstep(I1{}, SN{}, I0{}, I1{}, STAG, kt + 2);
+    // stage kt's buffers are free: its X buffer takes the W tile of stage kt + 2; second k-step
+    // from registers while the first fragments of stage kt + 1 are read
+    kstep(I1{}, xn, wn_, I0{}, I1{}, xb, kt + 2);
   };
 
-  // prologue: both stage buffers requested, the first one waited for
-  {
-    const uint32_t swv = (uint32_t)wave * 1024u;
+  // prologue: stages kb and kb + 1 requested, the first one waited for
 #pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-      unsigned char* const st = s2 ? st1 : st0;
-      const int ktc = min(kb + s2, ke - 1);
+  for (int i = 0; i < 8; ++i) {
+    load_x(tb0, kb, i);
+    load_w(tb1, kb, i);
+  }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void*)(st + (4 * i + wave) * 1024), 16, x_voff[i],
-                                                 (uint32_t)ktc * DG_ROW_BYTES, 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void*)(st + DG_OP_BYTES + (4 * i + wave) * 1024), 16, w_voff,
-                                                 (uint32_t)ktc * DG_OP_BYTES + swv + (uint32_t)i * 4096u, 0, 0);
-      }
-    }
+  for (int i = 0; i < 8; ++i) {
+    load_x(tb2, kb + 1, i);
+    load_w(tb3, kb + 1, i);
   }
   dg_wait_and_barrier<16>();
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    wf[0][i] = *reinterpret_cast<const h8*>(st0 + 16 * i * DG_ROW_BYTES + fw_off[0]);
-    xf[0][i] = *reinterpret_cast<const h8*>(st0 + 16 * i * DG_ROW_BYTES + fx_off[0]);
+    wf[0][i] = *reinterpret_cast<const h8*>(tb1 + 16 * i * DG_ROW_BYTES + fw_off[0]);
+    xf[0][i] = *reinterpret_cast<const h8*>(tb0 + 16 * i * DG_ROW_BYTES + fx_off[0]);
   }
   __builtin_amdgcn_sched_barrier(0);
   int kt = kb;
-  for (int full = (ke - kb) / 2; full > 0; --full, kt += 2) {
-    body(I0{}, kt);
-    body(I1{}, kt + 1);
+  for (int full = (ke - kb) / 5; full > 0; --full, kt += 5) {
+    body(std::integral_constant<int, 0>{}, kt);
+    body(std::integral_constant<int, 1>{}, kt + 1);
+    body(std::integral_constant<int, 2>{}, kt + 2);
+    body(std::integral_constant<int, 3>{}, kt + 3);
+    body(std::integral_constant<int, 4>{}, kt + 4);
   }
-  if (kt < ke) body(I0{}, kt);
+  // the stages left over when the count is not a multiple of five
+  if (kt < ke) {
+    body(std::integral_constant<int, 0>{}, kt);
+    if (kt + 1 < ke) {
+      body(std::integral_constant<int, 1>{}, kt + 1);
+      if (kt + 2 < ke) {
+        body(std::integral_constant<int, 2>{}, kt + 2);
+        if (kt + 3 < ke) body(std::integral_constant<int, 3>{}, kt + 3);
+      }
+    }
+  }
   // no load may still be writing this workgroup's LDS when it is handed to the next one; the
   // last MFMAs have left the pipe before their results are read (they are asm statements, for
   // which the compiler inserts no wait states)
