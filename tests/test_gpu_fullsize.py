@@ -77,6 +77,57 @@ def test_full_size_dequantize_rows_against_the_oracle(sba, gpu, name, K, N):
     assert bad.size == 0, f"{name}: first mismatches (sample row, column) {bad[:5].tolist()} of rows {rows}"
 
 
+def _one_hot_rows(K, gpu, seed, n):
+    """n row indices of K: first / last rows, first / last 128-row chunk, both sides of group
+    boundaries, the tail-step rows of a 231-chunk layer, and a random sample."""
+    rows = [0, 1, 31, 32, 127, 128, K - 129, K - 128, K - 97, K - 33, K - 32, K - 1]
+    rows += np.random.default_rng(seed).integers(0, K, n - len(rows)).tolist()
+    return sorted(set(int(r) for r in rows))
+
+
+@pytest.mark.parametrize("name,K,N", LAYERS)
+def test_full_size_gemm_one_hot_rows_against_the_oracle(sba, gpu, name, K, N):
+    """A second anchor of the full-size GEMM checks that does not pass through the dequantize
+    kernel: with a one-hot activation row e_k the skinny kernel returns row k of the dequantised
+    weights exactly, so sixteen such rows per call (M = 16) must equal the oracle's dequantize of
+    those rows bit for bit."""
+    qw, sc, qz, _ = _weights(K, N, gpu, 6)
+    rows = _one_hot_rows(K, gpu, K + N, 32)
+    for r0 in range(0, len(rows), 16):
+        ks = rows[r0:r0 + 16]
+        x = torch.zeros((len(ks), K), dtype=torch.float16, device=gpu)
+        x[torch.arange(len(ks), device=gpu), torch.tensor(ks, device=gpu)] = 1.0
+        y = sba.awq_gemm(x, qw, sc, qz, 0).cpu().numpy()
+        ridx = torch.tensor(ks, device=gpu)
+        gidx = ridx // 128
+        want = awq_ref.dequantize(qw[ridx].cpu().numpy(), sc[gidx].cpu().numpy(), qz[gidx].cpu().numpy(), 1)
+        bad = np.argwhere(y.view(np.uint16) != want.view(np.uint16))
+        assert bad.size == 0, f"{name}: first mismatches (row of the call, column) {bad[:5].tolist()} for k = {ks}"
+
+
+@pytest.mark.parametrize("name,K,N", LAYERS)
+def test_full_size_prefill_one_hot_rows_against_the_oracle(sba, gpu, name, K, N):
+    """The same anchor for the many-row path (panel pass + dense kernel at 2048 rows): a one-hot
+    row times exact fp16 weights is exact in the matrix pipe, so rows of a 2048-row call that are
+    one-hot must equal the oracle's dequantised rows bit for bit, wherever they sit in the call
+    (first / last row tile, next to random rows)."""
+    qw, sc, qz, g = _weights(K, N, gpu, 7)
+    M = 2048
+    ks = _one_hot_rows(K, gpu, 3 * K + N, 24)
+    at = np.random.default_rng(N).choice(np.arange(1, M - 1), size=len(ks), replace=False)
+    at[:2] = (0, M - 1)
+    x = torch.randn((M, K), device=gpu, generator=g).half()
+    x[torch.tensor(at, device=gpu)] = 0
+    x[torch.tensor(at, device=gpu), torch.tensor(ks, device=gpu)] = 1.0
+    y = sba.awq_gemm(x, qw, sc, qz, 0)
+    ridx = torch.tensor(ks, device=gpu)
+    gidx = ridx // 128
+    want = awq_ref.dequantize(qw[ridx].cpu().numpy(), sc[gidx].cpu().numpy(), qz[gidx].cpu().numpy(), 1)
+    got = y[torch.tensor(at, device=gpu)].cpu().numpy()
+    bad = np.argwhere(got.view(np.uint16) != want.view(np.uint16))
+    assert bad.size == 0, f"{name}: first mismatches (sample, column) {bad[:5].tolist()}"
+
+
 PREFILL_POINTS = [(n, K, N, M) for (n, K, N) in LAYERS for M in (512, 2048, 8192)]
 
 
