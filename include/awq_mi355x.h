@@ -41,7 +41,7 @@ typedef enum awqmi_status {
   AWQMI_SCRATCH_LIMIT = 8        /* awqmi_gemm_f16_noalloc: needs > AWQMI_STATIC_SCRATCH_BYTES */
 } awqmi_status;
 
-#define AWQMI_VERSION 201        /* major*10000 + minor*100 + patch */
+#define AWQMI_VERSION 300        /* major*10000 + minor*100 + patch */
 #define AWQMI_MOE_TILE_M 16      /* default rows per sorted-token block (32 also accepted)  */
 #define AWQMI_MAX_SPLIT_K 64
 #define AWQMI_MAX_EXPERTS 1024
@@ -112,8 +112,9 @@ int awqmi_dequantize_ld_f16(const int32_t* qweight, int ldw, const void* scales_
 /* awqmi_gemm_f16 for callers that cannot allocate or carry a workspace: code under HIP graph
  * capture that has no buffer of its own, tight serving loops, harnesses that forbid hipMalloc.
  * It has no counterpart in the harness or in vLLM's op surface (vLLM's awq_gemm allocates its
- * split-K buffer per call through torch).  Same arguments as awqmi_gemm_f16 minus the
- * workspace; the split-K arrival counters and fp32 partial tiles live in a static device array
+ * split-K buffer per call through torch).  Same arguments as awqmi_gemm_ld_f16 minus the
+ * workspace (ldw = words between consecutive rows of qweight; 0 or N / 8 for a contiguous tensor, more
+ * for the row-padded layout AWQLinearMethod keeps after loading); the split-K arrival counters and fp32 partial tiles live in a static device array
  * of AWQMI_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process
  * ends), and results are bit-identical to awqmi_gemm_f16 with a zeroed workspace of that many
  * bytes.  The call allocates and frees nothing.
@@ -131,7 +132,7 @@ int awqmi_dequantize_ld_f16(const int32_t* qweight, int ldw, const void* scales_
  *   - The device address of the array is looked up on the first call on each GPU (or by
  *     awqmi_init() with that GPU current); the stream must belong to the current device. */
 #define AWQMI_STATIC_SCRATCH_BYTES (AWQMI_WS_COUNTER_BYTES + (16u << 20))
-int awqmi_gemm_f16_noalloc(const void* x_f16, const int32_t* qweight, const void* scales_f16,
+int awqmi_gemm_f16_noalloc(const void* x_f16, const int32_t* qweight, int ldw, const void* scales_f16,
                            const int32_t* qzeros, void* y_f16, int M, int K, int N, int group,
                            int split_k, void* stream);
 

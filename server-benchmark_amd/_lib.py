@@ -25,8 +25,8 @@ SIGNATURES = {
                                   c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "awqmi_dequantize_ld_f16": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                         c_void_p]),
-    "awqmi_gemm_f16_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                                       c_int, c_void_p]),
+    "awqmi_gemm_f16_noalloc": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                       c_int, c_int, c_void_p]),
     "awqmi_moe_topk_softmax_f32": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "awqmi_moe_topk_f32": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, ctypes.c_float, c_void_p,
                                    c_void_p, c_void_p]),

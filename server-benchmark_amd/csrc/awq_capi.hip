@@ -270,8 +270,10 @@ int mfma_pick_rows(int M, int K, int N) {
 // needs one).
 static int ensure_kernel_attributes() {
   static std::atomic<bool> done[MAX_DEVICES];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) dev = 0;
+  int dev = -1;
+  const hipError_t ge = hipGetDevice(&dev);
+  if (ge != hipSuccess) { t_last_hip_error = (int)ge; return AWQMI_LAUNCH_FAILED; }
+  if (dev < 0 || dev >= MAX_DEVICES) return AWQMI_BAD_ARGUMENT;
   if (done[dev].load(std::memory_order_acquire)) return AWQMI_OK;
   const void* mfma[] = {
       reinterpret_cast<const void*>(awq_gemm_mfma_kernel<true, 1, 8>), reinterpret_cast<const void*>(awq_gemm_mfma_kernel<false, 1, 8>),
@@ -649,15 +651,15 @@ int awqmi_gemm_ld_f16(const void* x, const int32_t* qweight, int ldw, const void
   return launch_status();
 }
 
-int awqmi_gemm_f16_noalloc(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+int awqmi_gemm_f16_noalloc(const void* x, const int32_t* qweight, int ldw, const void* scales, const int32_t* qzeros,
                            void* y, int M, int K, int N, int group, int split_k, void* stream) {
   void* ptr = nullptr;
   bool first = false;
   if (const int rc = static_scratch_ptr(&ptr, &first)) return rc;
-  // exactly awqmi_gemm_f16 with this GPU's static array as the workspace (it validates before
+  // exactly awqmi_gemm_ld_f16 with this GPU's static array as the workspace (it validates before
   // it launches, so a skinny call whose split-K partial tiles do not fit launches nothing)
-  const int rc = awqmi_gemm_f16(x, qweight, scales, qzeros, y, ptr, AWQMI_STATIC_SCRATCH_BYTES, M, K, N, group,
-                                split_k, stream);
+  const int rc = awqmi_gemm_ld_f16(x, qweight, ldw == 0 ? N / 8 : ldw, scales, qzeros, y, ptr, AWQMI_STATIC_SCRATCH_BYTES,
+                                   M, K, N, group, split_k, stream);
   return rc == AWQMI_WORKSPACE_TOO_SMALL ? AWQMI_SCRATCH_LIMIT : rc;
 }
 

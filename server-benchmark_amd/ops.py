@@ -10,6 +10,8 @@ ROCm device; torch is used for memory and streams only.
 """
 from __future__ import annotations
 
+import warnings
+
 import torch
 
 from . import _lib
@@ -18,6 +20,7 @@ MOE_TILE_M = 16
 _WS_COUNTER_BYTES = 65536
 _workspaces: dict = {}
 _retired: list = []      # outgrown workspaces, kept because captured graphs may still point at them
+_warned_split_k_iters = False
 _gemm_ws_bytes: dict = {}  # (M, K, N, split) -> awqmi_gemm_workspace_bytes, asked once per shape
 DEV_VARIANT_NO_DENSE = 1 << 25   # development variant bits of awq_gemm (include/awq_mi355x_dev.h)
 DEV_VARIANT_DENSE = 1 << 26
@@ -154,6 +157,11 @@ def awq_gemm(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
     workgroups from the shape.  force_split_k (1 .. 64) forces a split-K factor for the skinny
     kernel; tests and sweeps use it.  _dev_variant routes the call through the library's
     development entry point (single launch rules switched off or forced)."""
+    global _warned_split_k_iters
+    if split_k_iters not in (0, 8) and not _warned_split_k_iters:
+        _warned_split_k_iters = True
+        warnings.warn(f"awq_gemm: split_k_iters={split_k_iters} is ignored (the library picks the split from the "
+                      "shape); pass force_split_k= to force a factor", stacklevel=2)
     _need(input, "input", torch.float16, 2)
     ldw = _need_qweight(qweight)
     _need(scales, "scales", torch.float16, 2)
@@ -195,14 +203,21 @@ def awq_gemm(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
     return out
 
 
+_noalloc_last_stream: dict = {}   # device index -> stream of the last awq_gemm_noalloc call
+
+
 def awq_gemm_noalloc(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, qzeros: torch.Tensor,
                      out: torch.Tensor, force_split_k: int | None = None) -> torch.Tensor:
     """awq_gemm into a caller-provided `out` through the library's allocation-free entry point:
     split-K counters and partial tiles live in a static device array inside the library, so
-    neither this wrapper nor the library allocates.  All such calls on one GPU share that array
-    and must not overlap in time.  Raises ValueError when the call's split-K tiles do not fit."""
+    neither this wrapper nor the library allocates.  qweight may be contiguous or row-padded (as
+    AWQLinearMethod holds it after loading).  All such calls on one GPU share that array and must
+    not overlap in time: when a call arrives on another stream than the previous one on that GPU,
+    the wrapper first waits on the host for the previous stream (and refuses to do so inside a
+    stream capture, where it cannot wait: callers on several streams use awq_gemm, whose workspace
+    is per stream).  Raises ValueError when the call's split-K tiles do not fit."""
     _need(input, "input", torch.float16, 2)
-    _need(qweight, "qweight", torch.int32, 2)
+    ldw = _need_qweight(qweight)
     _need(scales, "scales", torch.float16, 2)
     _need(qzeros, "qzeros", torch.int32, 2)
     _need(out, "out", torch.float16, 2)
@@ -213,9 +228,18 @@ def awq_gemm_noalloc(input: torch.Tensor, qweight: torch.Tensor, scales: torch.T
     if M == 0:
         return out
     split = 0 if force_split_k is None else max(0, min(int(force_split_k), 64))
-    st = _lib.load().awqmi_gemm_f16_noalloc(input.data_ptr(), qweight.data_ptr(), scales.data_ptr(),
-                                            qzeros.data_ptr(), out.data_ptr(), M, K, N, G, split,
-                                            _stream_ptr(input.device))
+    dev = input.device.index if input.device.index is not None else torch.cuda.current_device()
+    stream = _stream_ptr(input.device)
+    last = _noalloc_last_stream.get(dev)
+    if last is not None and last != stream:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("awq_gemm_noalloc: the previous call on this GPU ran on another stream and this one is "
+                               "being captured; the calls share one static scratch array and must be serialised "
+                               "(use awq_gemm, whose workspace is per stream)")
+        torch.cuda.ExternalStream(last, device=input.device).synchronize()
+    _noalloc_last_stream[dev] = stream
+    st = _lib.load().awqmi_gemm_f16_noalloc(input.data_ptr(), qweight.data_ptr(), ldw, scales.data_ptr(),
+                                            qzeros.data_ptr(), out.data_ptr(), M, K, N, G, split, stream)
     _lib.check(st, "awq_gemm_noalloc")
     return out
 

@@ -97,18 +97,35 @@ def _register_quant_config() -> bool:
     cls = make_vllm_config_class()
     table = getattr(quant, "_CUSTOMIZED_METHOD_TO_QUANT_CONFIG", None)
     names = getattr(quant, "QUANTIZATION_METHODS", None)
+    registered = False
     if isinstance(table, dict):
         table["awq"] = cls
         if isinstance(names, list) and "awq" not in names:
             names.append("awq")
+        registered = True
+    else:
+        deco = getattr(quant, "register_quantization_config", None)
+        if callable(deco):
+            try:
+                deco("awq")(cls)
+                registered = True
+            except ValueError:
+                pass
+    if registered:
+        # what vLLM hands out for the name must now be this class; a registry that resolves the
+        # name some other way would leave the server on its own kernels without a word
+        getter = getattr(quant, "get_quantization_config", None)
+        if callable(getter):
+            try:
+                got = getter("awq")
+            except Exception as e:           # noqa: BLE001 - any failure of the lookup is reported, not raised
+                got = e
+            if got is not cls:
+                warnings.warn(f"server_benchmark_amd: registered the `awq` config, but vLLM's "
+                              f"get_quantization_config('awq') returns {got!r}; linear and fused-MoE layers "
+                              "may stay on vLLM's kernels (the two AWQ ops are rebound either way)")
+                return False
         return True
-    deco = getattr(quant, "register_quantization_config", None)
-    if callable(deco):
-        try:
-            deco("awq")(cls)
-            return True
-        except ValueError:
-            pass
     warnings.warn("server_benchmark_amd: vLLM's quantization registry does not look as expected; only the two "
                   "AWQ ops were rebound (prefill >= 256 rows and fused-MoE layers stay on vLLM's kernels)")
     return False

@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol(lib):
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
     assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
-    assert lib.awqmi_version() == 201
+    assert lib.awqmi_version() == 300
 
 
 def test_status_strings(lib):
@@ -482,6 +482,25 @@ def test_vllm_plugin_registers_the_awq_method_for_linear_and_moe_layers(sba, mon
     assert tuple(seen["w13"]) == (4, 256, 32) and tuple(seen["w2"]) == (4, 128, 32)
     with pytest.raises(NotImplementedError):
         method.apply(moe_layer, x, lg, 2, True, apply_router_weight_on_input=True)
+
+
+def test_vllm_plugin_checks_what_the_registry_hands_out(sba, monkeypatch):
+    """After writing the table the plugin asks vLLM for the `awq` config: the registered class is a
+    success, anything else (a registry that resolves built-in names first) is warned about and not
+    reported as registered."""
+    import importlib
+    plugin = importlib.import_module(sba.__name__ + ".vllm_plugin")
+    mods = _fake_vllm(monkeypatch)
+    quant = mods["vllm.model_executor.layers.quantization"]
+    quant.get_quantization_config = lambda name: quant._CUSTOMIZED_METHOD_TO_QUANT_CONFIG[name]
+    assert "quantization:awq" in plugin.register()
+
+    class BuiltInAWQ:
+        pass
+
+    quant.get_quantization_config = lambda name: BuiltInAWQ
+    with pytest.warns(UserWarning, match="get_quantization_config"):
+        assert "quantization:awq" not in plugin.register()
 
 
 def test_create_weights_uses_vllm_parameter_classes_inside_vllm(sba, monkeypatch):

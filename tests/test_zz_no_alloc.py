@@ -37,7 +37,7 @@ def _both(lib, gpu, M, K, N, G, split, seed):
     torch.cuda.synchronize()
     print(f"[noalloc] M={M} K={K} N={N} G={G} split={split} needs {need} scratch bytes", flush=True)
     before = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
-    rc = lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), y_na.data_ptr(),
+    rc = lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qw.data_ptr(), 0, sc.data_ptr(), qz.data_ptr(), y_na.data_ptr(),
                                     M, K, N, G, split, st)
     assert rc == 0, lib.awqmi_status_string(rc).decode()
     torch.cuda.synchronize()
@@ -85,16 +85,16 @@ def test_noalloc_gemm_refuses_what_does_not_fit(gpu):
     st = torch.cuda.current_stream().cuda_stream
     # a forced split of 64 on this width wants 64 x 32 x 8192 fp32 partials = 64 MiB
     assert lib.awqmi_gemm_workspace_bytes(M, K, N, 64) > STATIC_BYTES
-    rc = lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), y.data_ptr(),
+    rc = lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qw.data_ptr(), 0, sc.data_ptr(), qz.data_ptr(), y.data_ptr(),
                                     M, K, N, G, 64, st)
     assert rc == SCRATCH_LIMIT
     assert "static" in lib.awqmi_status_string(rc).decode()
     torch.cuda.synchronize()
     assert not y.any()                      # nothing was launched
     # ordinary validation still comes first
-    assert lib.awqmi_gemm_f16_noalloc(0, qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), y.data_ptr(),
+    assert lib.awqmi_gemm_f16_noalloc(0, qw.data_ptr(), 0, sc.data_ptr(), qz.data_ptr(), y.data_ptr(),
                                       M, K, N, G, 0, st) == 6
-    assert lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), y.data_ptr(),
+    assert lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qw.data_ptr(), 0, sc.data_ptr(), qz.data_ptr(), y.data_ptr(),
                                       M, K, N + 4, G, 0, st) == 1
 
 
@@ -111,7 +111,7 @@ def test_noalloc_gemm_replays_from_a_captured_graph(gpu):
     y_graph = torch.zeros((M, N), dtype=torch.float16, device=gpu)
 
     def call(y, stream):
-        rc = lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), y.data_ptr(),
+        rc = lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qw.data_ptr(), 0, sc.data_ptr(), qz.data_ptr(), y.data_ptr(),
                                         M, K, N, G, 0, stream)
         assert rc == 0, lib.awqmi_status_string(rc).decode()
 
@@ -132,3 +132,31 @@ def test_noalloc_gemm_replays_from_a_captured_graph(gpu):
             other, _ = _both(lib, gpu, 3, 1024, 512, 128, 4, 12)       # eager calls on the same array in between
             assert torch.isfinite(other).all()
     torch.cuda.current_stream().wait_stream(s)
+
+
+def test_noalloc_gemm_takes_the_methods_row_padded_qweight(gpu):
+    """The layout AWQLinearMethod keeps after loading (rows one 128-byte line further apart) through
+    the allocation-free entry point and through its Python wrapper: the bits of the contiguous
+    tensor through awqmi_gemm_f16, on two calls in a row (the second with fewer rows)."""
+    from server_benchmark_amd import _lib, ops
+    lib = _lib.load()
+    assert lib.awqmi_init() == 0
+    K, N, G = 1024, 8192, 128
+    for M in (16, 3):
+        x, qw, sc, qz = _case(M, K, N, G, gpu, 40 + M)
+        qwp = ops.pad_qweight_rows(qw)
+        assert not qwp.is_contiguous() and qwp.stride(0) == N // 8 + 32
+        ws = torch.zeros(STATIC_BYTES, dtype=torch.uint8, device=gpu)
+        st = torch.cuda.current_stream().cuda_stream
+        y_ws = torch.empty((M, N), dtype=torch.float16, device=gpu)
+        assert lib.awqmi_gemm_f16(x.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), y_ws.data_ptr(),
+                                  ws.data_ptr(), ws.numel(), M, K, N, G, 0, st) == 0
+        y_c = torch.empty_like(y_ws)
+        assert lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qwp.data_ptr(), qwp.stride(0), sc.data_ptr(), qz.data_ptr(),
+                                          y_c.data_ptr(), M, K, N, G, 0, st) == 0
+        y_py = ops.awq_gemm_noalloc(x, qwp, sc, qz, torch.empty_like(y_ws))
+        torch.cuda.synchronize()
+        assert torch.equal(y_ws, y_c) and torch.equal(y_ws, y_py)
+    # a pitch that is no multiple of 16 bytes is refused before anything is launched
+    assert lib.awqmi_gemm_f16_noalloc(x.data_ptr(), qw.data_ptr(), N // 8 + 1, sc.data_ptr(), qz.data_ptr(),
+                                      y_c.data_ptr(), M, K, N, G, 0, st) != 0
