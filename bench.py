@@ -103,6 +103,12 @@ def main():
                          "decode sweep twice (direct launches) plus four 256 MiB device copies "
                          "(calibration of FETCH_SIZE / WRITE_SIZE).  prefill: awq_gemm at o_proj, "
                          "M=8192, three times.  moe: the Qwen3-30B-A3B MoE block at T=512, five times")
+    ap.add_argument("--probe", choices=("hbm-stream", "mfma"), default=None,
+                    help="measure a ceiling instead of the benchmark and print it as JSON.  hbm-stream: the skinny "
+                         "kernel's weight access pattern with the arithmetic removed over the four 72B qweight "
+                         "matrices (four rotating copies each, so every launch reads HBM), plus a plain linear read of "
+                         "1 GiB.  mfma: a bare loop of fp16 MFMAs on random operands, 60 launches of about 25 ms per "
+                         "instruction shape (what the matrix pipe sustains under the power limit)")
     ap.add_argument("--pmc-data", choices=("random", "const"), default="random",
                     help="with --pmc-target prefill: random operands (the benchmark's data) or the same value in "
                          "every weight, zero point, scale and activation (no operand bit toggles in the matrix pipe)")
@@ -176,6 +182,98 @@ def main():
     step_bytes = sum(workloads.linear_bytes(M, K, N, G) for _, K, N in layers for M in Ms)
     n_launch = len(layers) * len(Ms)
 
+    if args.probe == "hbm-stream":
+        sp = torch.cuda.current_stream().cuda_stream
+        res = {"probe": "hbm-stream", "peak_GBps": HBM_PEAK_GBS, "points": []}
+        sink = torch.empty(1 << 20, dtype=torch.int32, device=dev)
+        for name, K, N in layers:
+            parts = lib.awqmi_gemm_auto_split_k(1, K, N, G)
+            copies = [W[name][c][0] for c in range(NCOPY)]
+            def run(c):
+                st = lib.awqmi_dev_stream_probe(copies[c % NCOPY].data_ptr(), sink.data_ptr(), 0, K, N, parts, 0, sp)
+                if st != 0:
+                    raise RuntimeError(lib.awqmi_status_string(st).decode())
+            # the other layers' copies between two launches flush the last-level cache, as in the sweep
+            evs = []
+            for r in range(40):
+                for oname, oK, oN in layers:
+                    if oname != name:
+                        lib.awqmi_dev_stream_probe(W[oname][r % NCOPY][0].data_ptr(), sink.data_ptr(), 0, oK, oN,
+                                                   lib.awqmi_gemm_auto_split_k(1, oK, oN, G), 0, sp)
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                run(r)
+                b.record()
+                evs.append((a, b))
+            torch.cuda.synchronize()
+            ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs[8:])
+            med = ts[len(ts) // 2]
+            nbytes = K * N // 2
+            res["points"].append({"pattern": "skinny kernel's qweight reads", "layer": name, "K": K, "N": N, "parts": parts,
+                                  "workgroups": (N // 256) * parts, "bytes": nbytes, "us": round(med, 2),
+                                  "GBps": round(nbytes / med / 1e3, 1), "frac_hbm": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)})
+            log(f"   stream probe {name:13s} {med:8.2f} us  {nbytes / med / 1e3:8.1f} GB/s")
+            # the same bytes read linearly (what a layout made for streaming could reach at this size)
+            evs = []
+            nlin = nbytes // 1024 * 1024
+            for r in range(40):
+                for oname, oK, oN in layers:
+                    if oname != name:
+                        lib.awqmi_dev_stream_probe(W[oname][r % NCOPY][0].data_ptr(), sink.data_ptr(), 0, oK, oN,
+                                                   lib.awqmi_gemm_auto_split_k(1, oK, oN, G), 0, sp)
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                st = lib.awqmi_dev_stream_probe(copies[r % NCOPY].data_ptr(), sink.data_ptr(), 1, 0, 0, 1, nlin, sp)
+                b.record()
+                assert st == 0
+                evs.append((a, b))
+            torch.cuda.synchronize()
+            ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs[8:])
+            med = ts[len(ts) // 2]
+            res["points"].append({"pattern": "linear, 1 KiB per wave instruction", "layer": name, "bytes": nlin,
+                                  "workgroups": 256, "us": round(med, 2), "GBps": round(nlin / med / 1e3, 1),
+                                  "frac_hbm": round(nlin / med / 1e3 / HBM_PEAK_GBS, 4)})
+            log(f"   stream probe {name:13s} {med:8.2f} us  {nlin / med / 1e3:8.1f} GB/s  (the same bytes, linear)")
+        big = [torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(2)]
+        evs = []
+        for r in range(20):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            st = lib.awqmi_dev_stream_probe(big[r % 2].data_ptr(), sink.data_ptr(), 1, 0, 0, 1, 1 << 30, sp)
+            b.record()
+            assert st == 0
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs[4:])
+        med = ts[len(ts) // 2]
+        res["points"].append({"pattern": "linear, 1 KiB per wave instruction", "bytes": 1 << 30, "us": round(med, 2),
+                              "GBps": round((1 << 30) / med / 1e3, 1), "frac_hbm": round((1 << 30) / med / 1e3 / HBM_PEAK_GBS, 4)})
+        log(f"   stream probe linear 1 GiB  {med:8.2f} us  {(1 << 30) / med / 1e3:8.1f} GB/s")
+        print(json.dumps(res))
+        return
+    if args.probe == "mfma":
+        sp = torch.cuda.current_stream().cuda_stream
+        src = torch.randn(8 << 20, device=dev, generator=gen).to(torch.float16)      # 16 MiB of N(0, 1) fp16 values
+        sink = torch.empty(65536, dtype=torch.float32, device=dev)
+        res = {"probe": "mfma", "peak_TFLOPs": MFMA_FP16_PEAK_TFLOPS, "points": []}
+        for shape, iname in ((0, "v_mfma_f32_32x32x16_f16"), (1, "v_mfma_f32_16x16x32_f16")):
+            iters = 20000
+            fl = 256 * 4 * iters * 2097152.0
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(61)]
+            evs[0].record()
+            for i in range(60):
+                st = lib.awqmi_dev_mfma_probe(src.data_ptr(), sink.data_ptr(), shape, iters, sp)
+                assert st == 0
+                evs[i + 1].record()
+            torch.cuda.synchronize()
+            tf = [fl / (evs[i].elapsed_time(evs[i + 1]) * 1e-3) / 1e12 for i in range(60)]
+            settled = sorted(tf[20:])[20]
+            res["points"].append({"instruction": iname, "operands": "random N(0,1) fp16 in registers, two alternating sets",
+                                  "TFLOPs_first_launch": round(tf[0], 1), "TFLOPs_sustained": round(settled, 1),
+                                  "frac_mfma": round(settled / MFMA_FP16_PEAK_TFLOPS, 4), "launch_ms": round(fl / settled / 1e9, 2)})
+            log(f"   mfma probe {iname}: first launch {tf[0]:.0f}, sustained {settled:.0f} TFLOP/s")
+        print(json.dumps(res))
+        return
     if args.pmc_target == "prefill":
         name, K, N = layers[1]
         qw, sc, qz = W[name][0]
@@ -184,14 +282,18 @@ def main():
             qw, sc, qz = torch.full_like(qw, 0x77777777), torch.full_like(sc, 0.01), torch.full_like(qz, 0x33333333)
             xp.fill_(1.0)
         yp = torch.empty((8192, N), dtype=torch.float16, device=dev)
-        for _ in range(3):
-            st = lib.awqmi_gemm_ld_f16(xp.data_ptr(), qw.data_ptr(), qw.stride(0), sc.data_ptr(), qz.data_ptr(),
-                                       yp.data_ptr(), ws.data_ptr(), ws.numel(), 8192, K, N, G, 0,
-                                       torch.cuda.current_stream().cuda_stream)
-            assert st == 0
+        # twelve calls of the default rule (dequantise once + dense kernel at this row count), then
+        # twelve of the per-tile kernel through the development entry point, for a side-by-side record
+        for variant in (-1, 1 << 25):
+            for _ in range(12):
+                st = lib.awqmi_dev_gemm_f16(xp.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), yp.data_ptr(),
+                                            ws.data_ptr(), ws.numel(), 8192, K, N, G, 0,
+                                            torch.cuda.current_stream().cuda_stream, variant)
+                assert st == 0
         torch.cuda.synchronize()
-        log(f"[bench] pmc target: 3 x awq_gemm {name} M=8192 K={K} N={N} "
-            f"({workloads.linear_flops(8192, K, N)} flops each), {args.pmc_data} operands")
+        log(f"[bench] pmc target: awq_gemm {name} M=8192 K={K} N={N} ({workloads.linear_flops(8192, K, N)} flops each), "
+            f"{args.pmc_data} operands: 12 calls as awq_dequant_panel_kernel + awq_gemm_dense_kernel, then 12 calls as "
+            f"awq_gemm_mfma_kernel")
         return
     if args.pmc_target == "moe":
         mq = workloads.QWEN3_MOE

@@ -60,6 +60,22 @@ int awqmi_dev_last_gemm_form(void);
  * K-split partial tiles, fp16 panel); 0 when the shape cannot (K % 64 != 0). */
 size_t awqmi_dev_gemm_dense_workspace_bytes(int M, int K, int N);
 
+/* Measurement probes (no counterpart anywhere: they exist so that the ceilings the kernels are
+ * priced against are measured on the machine).
+ * awqmi_dev_stream_probe: a read-only pass with the arithmetic removed.  pattern 0 reads an int32
+ * [K, N / 8] matrix the way the skinny GEMM kernel reads qweight (workgroup = 256 columns x one
+ * of `parts` K ranges, one 128-byte line per row and 16 lanes, four 32-row steps in flight per
+ * wave; K % 128 == 0, N % 256 == 0, K / 128 >= 4 parts; `out` takes (N / 256) * parts * 256 words);
+ * pattern 1 reads total_bytes linearly (256 workgroups, 1 KiB per wave instruction, 16 KiB in
+ * flight per wave; `out` takes 65536 words).
+ * awqmi_dev_mfma_probe: 256 workgroups x 4 waves, each a bare loop of fp16 MFMAs over a 128 x 128
+ * accumulator tile with two alternating fragment sets taken from `src` (16 MiB of fp16 values);
+ * shape 0 = v_mfma_f32_32x32x16_f16, shape 1 = v_mfma_f32_16x16x32_f16; one iteration is 2097152
+ * flop per wave; `out` takes 65536 floats. */
+int awqmi_dev_stream_probe(const void* src, void* out, int pattern, int K, int N, int parts, size_t total_bytes,
+                           void* stream);
+int awqmi_dev_mfma_probe(const void* src, void* out, int shape, int iters, void* stream);
+
 int awqmi_dev_moe_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
                            const int32_t* qzeros, void* y_f16, const int32_t* sorted_token_ids,
                            const int32_t* expert_ids, const int32_t* num_tokens_post_padded,

@@ -17,6 +17,7 @@
 #include "awq_gemm_mfma.hpp"
 #include "awq_gemv.hpp"
 #include "awq_moe.hpp"
+#include "awq_probes.hpp"
 
 using namespace awqmi;
 
@@ -1184,6 +1185,41 @@ int awqmi_dev_gemm_f16(const void* x, const int32_t* qweight, const void* scales
 }
 
 int awqmi_dev_last_gemm_form(void) { return t_last_gemm_form; }
+
+int awqmi_dev_stream_probe(const void* src, void* out, int pattern, int K, int N, int parts, size_t total_bytes,
+                           void* stream) {
+  if (!src || !out) return AWQMI_NULL_POINTER;
+  if (!aligned16(src) || !aligned16(out)) return AWQMI_BAD_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  if (pattern == 0) {
+    // whole 128-byte lines per column block, whole 128-row chunks, at least one chunk per wave
+    if (K <= 0 || N <= 0 || K % 128 != 0 || N % 256 != 0 || parts < 1 || (K / 128) < 4 * parts) return AWQMI_BAD_SHAPE;
+    if ((size_t)(N / 256) * parts > 65535u * 4u) return AWQMI_BAD_SHAPE;
+    hipLaunchKernelGGL((awq_stream_probe_kernel<0>), dim3(N / 256, parts), dim3(256), 0, st,
+                       reinterpret_cast<const uint32_t*>(src), reinterpret_cast<uint32_t*>(out), K, N / 8, parts, (size_t)0);
+  } else if (pattern == 1) {
+    if (total_bytes < (1u << 20) || total_bytes % 1024 != 0) return AWQMI_BAD_SHAPE;
+    hipLaunchKernelGGL((awq_stream_probe_kernel<1>), dim3(256), dim3(256), 0, st, reinterpret_cast<const uint32_t*>(src),
+                       reinterpret_cast<uint32_t*>(out), 0, 0, 1, total_bytes);
+  } else {
+    return AWQMI_BAD_ARGUMENT;
+  }
+  return launch_status();
+}
+
+int awqmi_dev_mfma_probe(const void* src, void* out, int shape, int iters, void* stream) {
+  if (!src || !out) return AWQMI_NULL_POINTER;
+  if (!aligned16(src) || !aligned16(out)) return AWQMI_BAD_ALIGN;
+  if (iters <= 0 || (shape != 0 && shape != 1)) return AWQMI_BAD_ARGUMENT;
+  hipStream_t st = (hipStream_t)stream;
+  if (shape == 0)
+    hipLaunchKernelGGL((awq_mfma_probe_kernel<0>), dim3(256), dim3(256), 0, st, reinterpret_cast<const uint32_t*>(src),
+                       reinterpret_cast<float*>(out), iters);
+  else
+    hipLaunchKernelGGL((awq_mfma_probe_kernel<1>), dim3(256), dim3(256), 0, st, reinterpret_cast<const uint32_t*>(src),
+                       reinterpret_cast<float*>(out), iters);
+  return launch_status();
+}
 
 size_t awqmi_dev_gemm_dense_workspace_bytes(int M, int K, int N) {
   if (M <= 0 || K <= 0 || N <= 0 || K % 64 != 0) return 0;
