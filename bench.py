@@ -103,12 +103,14 @@ def main():
                          "decode sweep twice (direct launches) plus four 256 MiB device copies "
                          "(calibration of FETCH_SIZE / WRITE_SIZE).  prefill: awq_gemm at o_proj, "
                          "M=8192, three times.  moe: the Qwen3-30B-A3B MoE block at T=512, five times")
-    ap.add_argument("--probe", choices=("hbm-stream", "mfma"), default=None,
+    ap.add_argument("--probe", choices=("hbm-stream", "mfma", "decode-timeline"), default=None,
                     help="measure a ceiling instead of the benchmark and print it as JSON.  hbm-stream: the skinny "
                          "kernel's weight access pattern with the arithmetic removed over the four 72B qweight "
                          "matrices (four rotating copies each, so every launch reads HBM), plus a plain linear read of "
                          "1 GiB.  mfma: a bare loop of fp16 MFMAs on random operands, 60 launches of about 25 ms per "
-                         "instruction shape (what the matrix pipe sustains under the power limit)")
+                         "instruction shape (what the matrix pipe sustains under the power limit).  decode-timeline: "
+                         "per-workgroup time stamps at the phase boundaries of the skinny kernel for every layer of the "
+                         "sweep at M = 1 and 16 (where a launch's time goes)")
     ap.add_argument("--pmc-data", choices=("random", "const"), default="random",
                     help="with --pmc-target prefill: random operands (the benchmark's data) or the same value in "
                          "every weight, zero point, scale and activation (no operand bit toggles in the matrix pipe)")
@@ -249,6 +251,48 @@ def main():
         res["points"].append({"pattern": "linear, 1 KiB per wave instruction", "bytes": 1 << 30, "us": round(med, 2),
                               "GBps": round((1 << 30) / med / 1e3, 1), "frac_hbm": round((1 << 30) / med / 1e3 / HBM_PEAK_GBS, 4)})
         log(f"   stream probe linear 1 GiB  {med:8.2f} us  {(1 << 30) / med / 1e3:8.1f} GB/s")
+        print(json.dumps(res))
+        return
+    if args.probe == "decode-timeline":
+        sp = torch.cuda.current_stream().cuda_stream
+        phases = ["workgroup starts", "main loop left", "cross-wave LDS sum done", "partial stores acknowledged",
+                  "arrival counted", "last arriver: partials summed", "output stored, workgroup ends"]
+        res = {"probe": "decode-timeline", "unit": "us after the first workgroup's start; min / median / max over the "
+               "workgroups that reach the phase", "points": []}
+        for name, K, N in layers:
+            for M in (1, 16):
+                split = lib.awqmi_gemm_auto_split_k(M, K, N, G)
+                wgs = ((N // 8 + 31) // 32) * split
+                stamps = torch.zeros(wgs * 8, dtype=torch.int64, device=dev)
+                rows = None
+                for r in range(12):
+                    # the other layers in between, as in the sweep: every launch reads its weights from HBM
+                    for oname, oK, oN in layers:
+                        if oname != name:
+                            launch(oname, oK, oN, 16, r % NCOPY, sp)
+                    qw, sc, qz = W[name][r % NCOPY]
+                    stamps.zero_()
+                    st = lib.awqmi_dev_gemm_timeline_f16(X[name][M].data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(),
+                                                         Y[name][M].data_ptr(), ws.data_ptr(), ws.numel(), M, K, N, G, 0, sp,
+                                                         stamps.data_ptr(), stamps.numel() * 8)
+                    if st != 0:
+                        raise RuntimeError(lib.awqmi_status_string(st).decode())
+                    torch.cuda.synchronize()
+                    t = stamps.view(wgs, 8).cpu().double() / 100.0          # 100 MHz counter -> us
+                    t0 = float(t[:, 0].min())
+                    cur = []
+                    for k in range(7):
+                        v = t[:, k][t[:, k] > 0] - t0
+                        cur.append(None if v.numel() == 0 else
+                                   [round(float(v.min()), 2), round(float(v.median()), 2), round(float(v.max()), 2), int(v.numel())])
+                    if r >= 4:        # the first launches warm code and clocks
+                        rows = cur if rows is None else [a if b is None else [round((a[i] * (r - 4) + b[i]) / (r - 3), 2) for i in range(3)] + [b[3]]
+                                                         for a, b in zip(rows, cur)]
+                pt = {"layer": name, "M": M, "K": K, "N": N, "split_k": split, "workgroups": wgs,
+                      "phases": {phases[k]: rows[k] for k in range(7) if rows[k] is not None}}
+                res["points"].append(pt)
+                log(f"   timeline {name:13s} M={M:2d} split {split} ({wgs} workgroups): " +
+                    "; ".join(f"{phases[k]} {rows[k][0]:.2f}/{rows[k][1]:.2f}/{rows[k][2]:.2f}" for k in range(7) if rows[k] is not None))
         print(json.dumps(res))
         return
     if args.probe == "mfma":

@@ -76,6 +76,17 @@ int awqmi_dev_stream_probe(const void* src, void* out, int pattern, int K, int N
                            void* stream);
 int awqmi_dev_mfma_probe(const void* src, void* out, int shape, int iters, void* stream);
 
+/* awqmi_gemm_f16 for one decode-sized call (M <= 16) that also records, per workgroup, seven
+ * time stamps of a constant 100 MHz counter at the kernel's phase boundaries (stamps[8 w + k] for
+ * workgroup w = part * column_blocks + column_block: 0 start, 1 main loop left, 2 cross-wave sum
+ * in LDS done, 3 partial stores acknowledged, 4 arrival counted, 5 last arriver: partials summed,
+ * 6 output stored; 3 - 5 only in split-K launches, 5 - 6 only in the finishing workgroup).  The
+ * buffer must be zeroed by the caller and hold 8 words per workgroup. */
+int awqmi_dev_gemm_timeline_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
+                                const int32_t* qzeros, void* y_f16, void* workspace, size_t workspace_bytes,
+                                int M, int K, int N, int group, int split_k, void* stream,
+                                unsigned long long* stamps, size_t stamps_bytes);
+
 int awqmi_dev_moe_gemm_f16(const void* x_f16, const int32_t* qweight, const void* scales_f16,
                            const int32_t* qzeros, void* y_f16, const int32_t* sorted_token_ids,
                            const int32_t* expert_ids, const int32_t* num_tokens_post_padded,

@@ -56,6 +56,8 @@ for _name in ("awqmi_gemm_f16", "awqmi_moe_gemm_f16", "awqmi_fused_moe_routed_f1
 SIGNATURES["awqmi_dev_last_gemm_form"] = (c_int, [])
 SIGNATURES["awqmi_dev_gemm_dense_workspace_bytes"] = (c_size_t, [c_int, c_int, c_int])
 SIGNATURES["awqmi_dev_stream_probe"] = (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_size_t, c_void_p])
+SIGNATURES["awqmi_dev_gemm_timeline_f16"] = (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                                      c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t])
 SIGNATURES["awqmi_dev_mfma_probe"] = (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p])
 FORM_SKINNY, FORM_FUSED, FORM_DENSE, FORM_GENERIC = 1, 2, 3, 4   # awqmi_dev_last_gemm_form()
 

@@ -33,6 +33,8 @@ namespace {
 thread_local int t_last_hip_error = 0;
 // which kernel family the last awqmi_gemm_* call on this thread launched (awqmi_dev_last_gemm_form)
 thread_local int t_last_gemm_form = 0;
+// time-stamp buffer of the call in progress (awqmi_dev_gemm_timeline_f16 only; null otherwise)
+thread_local unsigned long long* t_trace = nullptr;
 
 // Launch-rule variant of the call in progress on this thread: -1 (every default) for the whole
 // public C ABI; the awqmi_dev_* entry points set it for the duration of their own call only, so
@@ -64,6 +66,7 @@ enum : int {
   VAR_NO_FOLDED_ROUTE = 1 << 24, // the one-call MoE block always routes in a launch of its own
   VAR_NO_DENSE = 1 << 25,        // awq_gemm never takes the dequantise-once form
   VAR_DENSE = 1 << 26,           // awq_gemm takes the dequantise-once form from 257 rows on (workspace permitting)
+  VAR_MOE_T32_WIDE = 1 << 27,    // 32-row MoE blocks in the two-words-per-lane form (one workgroup per CU)
 };
 inline bool variant_on(int bit) {
   return t_variant >= 0 && (t_variant & bit);
@@ -538,6 +541,7 @@ int awqmi_gemm_ld_f16(const void* x, const int32_t* qweight, int ldw, const void
                        : nullptr;
     p.K = K; p.N = N; p.NW = NW; p.ldw = ldw; p.G = G; p.ldy = N;
     p.split_k = split; p.ncb = ncb;
+    p.trace = t_trace;
     const dim3 grid(ncb, split, 1);
     // passes of up to 32 rows; each pass streams the weights once
     for (int r0 = 0; r0 < M; r0 += 32) {
@@ -864,7 +868,11 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   }
   const MoePlan pl = moe_plan(n_slots, E, K, N, tile_m, split_k);
   const int wpl = pl.wpl, ncb = pl.ncb, nblk = pl.nblk, split = pl.split;
-  if (tile_m == 32 && wpl != 2) return AWQMI_BAD_SHAPE;   // 32-row blocks need N % 16 == 0
+  // 32-row blocks: one packed word per lane, two column blocks of 128 per workgroup with two waves
+  // each (the accumulators of two row blocks then take the registers one row block takes with two
+  // words per lane, and two workgroups still fit a CU); needs an even chunk count, no K split
+  const bool t32_narrow = tile_m == 32 && split == 1 && (K / 128) % 2 == 0 && !variant_on(VAR_MOE_T32_WIDE);
+  if (tile_m == 32 && !t32_narrow && wpl != 2) return AWQMI_BAD_SHAPE;   // the wide form needs N % 16 == 0
   if (split > 1) {
     if (!workspace) return AWQMI_NULL_POINTER;
     if (!aligned16(workspace)) return AWQMI_BAD_ALIGN;
@@ -911,7 +919,9 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   const bool act_split = fuse_act && split > 1;
   p.act_split = act_split ? 1 : 0;
   const bool act_pair = fuse_act && split == 1;
-  const int ncg = act_pair ? ncb / 2 : (pair_cols ? (ncb + 1) / 2 : ncb);
+  const int ncb1 = (NW + 15) / 16;       // column blocks of 128 (one word per lane)
+  const int ncg = t32_narrow ? (ncb1 + 1) / 2 : (act_pair ? ncb / 2 : (pair_cols ? (ncb + 1) / 2 : ncb));
+  if (t32_narrow) p.ncb = ncb1;
   // runs of grp slots, dealt to the 8 XCDs in turn; the last deal may be partial
   const long long runs = (long long)(nblk / p.grp) * ncg * split;
   const dim3 grid((unsigned)((runs + 7) / 8 * 8 * p.grp));
@@ -950,6 +960,7 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   else if (ldsq) launch_gemv<2, 1, true, 4, 4, false, true>(p, grid, st);
   else if (act_pair) launch_gemv<2, 1, true, 2, 2, true>(p, grid, st);
   else if (act_split) launch_gemv<2, 1, true, 2>(p, grid, st);
+  else if (t32_narrow) launch_gemv<1, 2, true, 2, 2>(p, grid, st);
   else if (tile_m == 32) launch_gemv<2, 2, true>(p, grid, st);
   else if (wpl == 2 && variant_on(VAR_MOE_RING4)) launch_gemv<2, 1, true, 4>(p, grid, st);
   else if (pair_cols) launch_gemv<2, 1, true, 2, 2>(p, grid, st);
@@ -1185,6 +1196,22 @@ int awqmi_dev_gemm_f16(const void* x, const int32_t* qweight, const void* scales
 }
 
 int awqmi_dev_last_gemm_form(void) { return t_last_gemm_form; }
+
+int awqmi_dev_gemm_timeline_f16(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                                void* y, void* workspace, size_t workspace_bytes, int M, int K, int N, int group,
+                                int split_k, void* stream, unsigned long long* stamps, size_t stamps_bytes) {
+  if (!stamps) return AWQMI_NULL_POINTER;
+  if (M <= 0 || M > 16 || K <= 0 || N <= 0) return AWQMI_BAD_SHAPE;     // one dense skinny launch
+  const int G = norm_group(K, group);
+  if (check_awq_shape(K, N, G) != AWQMI_OK || !gemv_tiled_ok(K, G)) return AWQMI_BAD_SHAPE;
+  const int split = split_k > 0 ? split_k : pick_split_k(M, K, N, G, 1, true);
+  const size_t wgs = (size_t)((N / 8 + 16 * gemv_wpl(N) - 1) / (16 * gemv_wpl(N))) * split;
+  if (stamps_bytes < wgs * 8 * sizeof(unsigned long long)) return AWQMI_WORKSPACE_TOO_SMALL;
+  t_trace = stamps;
+  const int rc = awqmi_gemm_f16(x, qweight, scales, qzeros, y, workspace, workspace_bytes, M, K, N, group, split_k, stream);
+  t_trace = nullptr;
+  return rc;
+}
 
 int awqmi_dev_stream_probe(const void* src, void* out, int pattern, int K, int N, int parts, size_t total_bytes,
                            void* stream) {

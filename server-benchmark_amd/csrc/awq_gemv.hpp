@@ -60,6 +60,9 @@ struct GemvParams {
   int* r_sorted;           // out: 16 entries per block that runs
   int* r_experts;          // out: one per block that runs
   int* r_npp;              // out: 16 x blocks that run
+  // Dense launches only, null outside the timeline probe: eight time stamps per workgroup
+  // (constant-rate 100 MHz counter) at the phase boundaries of the kernel.
+  unsigned long long* trace;
 };
 
 typedef float f2 __attribute__((ext_vector_type(2)));
@@ -451,6 +454,15 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, h = lane >> 4;
   int cb = blockIdx.x, sp = blockIdx.y;
+  // phase stamps of the timeline probe: 0 start, 1 main loop left, 2 cross-wave sum done,
+  // 3 partial stores acknowledged, 4 arrival counted, 5 (last arriver) partials summed, 6 output stored
+  auto stamp = [&](int k) {
+    if constexpr (!MOE) {
+      if (p.trace && tid == 0)
+        p.trace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 8 + k] = __builtin_amdgcn_s_memrealtime();
+    }
+  };
+  stamp(0);
   int blk = 0;
   float row_tw = 1.f;   // MoE: routing weight of row tid (threads below TM), parked in s_tw after the loop
   const uint32_t* qw = p.qw;
@@ -608,6 +620,7 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
     const int c_end = (int)((pw + 1) * (unsigned)nchunks / parts);
     w.run(c_begin, c_end);
   }
+  stamp(1);
   if (LDSQ) __syncthreads();   // the cross-wave sum below reuses ring slots 0 and 1
   if (MOE && tid < TM) s_tw[tid] = row_tw;   // read behind the barriers of the cross-wave sum
 
@@ -723,6 +736,7 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
         }
     }
     __syncthreads();
+    if (mb == 0) stamp(2);
     if (split) {
       // fp32 partial tile of this workgroup.  Partials and the arrival counter go through
       // device-coherent accesses (they bypass the per-XCD L2 for other XCDs' data) instead of
@@ -741,12 +755,16 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
     }
     __syncthreads();
   }
-  if (!split) return;
+  if (!split) {
+    stamp(6);
+    return;
+  }
 
   // Ordering: every store of this workgroup has completed (vmcnt 0, then the barrier)
   // before its arrival is counted; whoever arrives last sums all partials in fixed order.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+  stamp(3);
   // fused activation: a gate block and its up block (half the column blocks further on) share
   // one counter, and the last of their 2 x split workgroups finishes both tiles
   const bool acts = MOE && MB == 1 && KW == 4 && !ACT && p.act_split;
@@ -756,6 +774,7 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
   const int arrivals = acts ? 2 * p.split_k : p.split_k;
   if (tid == 0) s_last = (atomicAdd(p.cnt + ctile, 1) == arrivals - 1);
   __syncthreads();
+  stamp(4);
   if (!s_last) return;
   const size_t sstride = ntiles * MB * TILE_F;
   // U pairs per thread x 8 parts per batch: 8 * U independent 8-byte loads in flight; parts
@@ -821,14 +840,16 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
       else finish(std::integral_constant<int, 8>{}, base, nelem);
     }
     __syncthreads();
+    if (mb == 0) stamp(5);
     emit(mb, rows, false);
     __syncthreads();
   }
+  stamp(6);
   if (tid == 0) __hip_atomic_store(p.cnt + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <int WPL, int GMODE, int MB, bool MOE, int RING = 4, int KW = 4, bool ACT = false, bool LDSQ = false>
-__global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || MB == 2) ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
+__global__ __launch_bounds__(256, ((RING == 4 && !LDSQ) || (MB == 2 && WPL == 2)) ? 1 : 2) void awq_gemv_kernel(const GemvParams p) {
   awq_gemv_body<WPL, GMODE, MB, MOE, RING, KW, ACT, LDSQ, false>(p);
 }
 
