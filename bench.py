@@ -85,11 +85,13 @@ def main():
     ap.add_argument("--split-k", type=int, default=0, help="0 = library heuristic")
     ap.add_argument("--variant", type=int, default=-1,
                     help="development: run the decode sweep through awqmi_dev_gemm_f16 with this launch-rule variant")
-    ap.add_argument("--rows", choices=("contiguous", "method"), default="contiguous",
-                    help="layout of the dense layers' qweight: contiguous as in the checkpoint (what the ops "
-                         "awq_gemm / awq_dequantize are handed by vLLM's own method), or as this package's "
-                         "AWQLinearMethod.process_weights_after_loading holds it (rows of N >= 8192 that are a "
-                         "multiple of 512 bytes get one 128-byte line of pitch more); the other layout's sweep is timed beside it")
+    ap.add_argument("--rows", choices=("contiguous", "method"), default="method",
+                    help="layout of the dense layers' qweight: as this package's "
+                         "AWQLinearMethod.process_weights_after_loading holds it, i.e. what the layer method's apply -- the "
+                         "path a served model takes -- multiplies by (rows of N >= 8192 that are a multiple of 512 bytes "
+                         "get one 128-byte line of pitch more; same values, same algorithmic bytes), or contiguous as in "
+                         "the checkpoint (what the bare ops awq_gemm / awq_dequantize are handed when only they are "
+                         "rebound under vLLM's own method); the other layout's sweep is timed beside it")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--decoder", action="store_true", help=argparse.SUPPRESS)   # kept for old command lines
@@ -188,54 +190,44 @@ def main():
         sp = torch.cuda.current_stream().cuda_stream
         res = {"probe": "hbm-stream", "peak_GBps": HBM_PEAK_GBS, "points": []}
         sink = torch.empty(1 << 20, dtype=torch.int32, device=dev)
+        def flush_cache(name, r):
+            # the other layers' copies between two timed launches, as in the sweep
+            for oname, oK, oN in layers:
+                if oname != name:
+                    lib.awqmi_dev_stream_probe(W[oname][r % NCOPY][0].data_ptr(), sink.data_ptr(), 1, 0, 0, 1,
+                                               oK * oN // 2 // 1024 * 1024, sp)
+
         for name, K, N in layers:
             parts = lib.awqmi_gemm_auto_split_k(1, K, N, G)
-            copies = [W[name][c][0] for c in range(NCOPY)]
-            def run(c):
-                st = lib.awqmi_dev_stream_probe(copies[c % NCOPY].data_ptr(), sink.data_ptr(), 0, K, N, parts, 0, sp)
-                if st != 0:
-                    raise RuntimeError(lib.awqmi_status_string(st).decode())
-            # the other layers' copies between two launches flush the last-level cache, as in the sweep
-            evs = []
-            for r in range(40):
-                for oname, oK, oN in layers:
-                    if oname != name:
-                        lib.awqmi_dev_stream_probe(W[oname][r % NCOPY][0].data_ptr(), sink.data_ptr(), 0, oK, oN,
-                                                   lib.awqmi_gemm_auto_split_k(1, oK, oN, G), 0, sp)
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                run(r)
-                b.record()
-                evs.append((a, b))
-            torch.cuda.synchronize()
-            ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs[8:])
-            med = ts[len(ts) // 2]
             nbytes = K * N // 2
-            res["points"].append({"pattern": "skinny kernel's qweight reads", "layer": name, "K": K, "N": N, "parts": parts,
-                                  "workgroups": (N // 256) * parts, "bytes": nbytes, "us": round(med, 2),
-                                  "GBps": round(nbytes / med / 1e3, 1), "frac_hbm": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)})
-            log(f"   stream probe {name:13s} {med:8.2f} us  {nbytes / med / 1e3:8.1f} GB/s")
-            # the same bytes read linearly (what a layout made for streaming could reach at this size)
-            evs = []
-            nlin = nbytes // 1024 * 1024
-            for r in range(40):
-                for oname, oK, oN in layers:
-                    if oname != name:
-                        lib.awqmi_dev_stream_probe(W[oname][r % NCOPY][0].data_ptr(), sink.data_ptr(), 0, oK, oN,
-                                                   lib.awqmi_gemm_auto_split_k(1, oK, oN, G), 0, sp)
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                st = lib.awqmi_dev_stream_probe(copies[r % NCOPY].data_ptr(), sink.data_ptr(), 1, 0, 0, 1, nlin, sp)
-                b.record()
-                assert st == 0
-                evs.append((a, b))
-            torch.cuda.synchronize()
-            ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs[8:])
-            med = ts[len(ts) // 2]
-            res["points"].append({"pattern": "linear, 1 KiB per wave instruction", "layer": name, "bytes": nlin,
-                                  "workgroups": 256, "us": round(med, 2), "GBps": round(nlin / med / 1e3, 1),
-                                  "frac_hbm": round(nlin / med / 1e3 / HBM_PEAK_GBS, 4)})
-            log(f"   stream probe {name:13s} {med:8.2f} us  {nlin / med / 1e3:8.1f} GB/s  (the same bytes, linear)")
+            contiguous = [W[name][c][0].contiguous() for c in range(NCOPY)]
+            padded = [ops.pad_qweight_rows(t) for t in contiguous]
+            forms = [("skinny kernel's reads, contiguous rows", 0, contiguous, None)]
+            if padded[0].stride(0) != contiguous[0].stride(0):
+                forms.append(("skinny kernel's reads, rows one 128-byte line further apart", 0, padded, None))
+            forms.append(("one contiguous run per wave", 1, contiguous, nbytes // 1024 * 1024))
+            for label, pattern, copies, linear_bytes in forms:
+                evs = []
+                for r in range(40):
+                    flush_cache(name, r)
+                    t = copies[r % NCOPY]
+                    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    a.record()
+                    st = lib.awqmi_dev_stream_probe(t.data_ptr(), sink.data_ptr(), pattern, K, N, parts,
+                                                    t.stride(0) if linear_bytes is None else linear_bytes, sp)
+                    b.record()
+                    if st != 0:
+                        raise RuntimeError(lib.awqmi_status_string(st).decode())
+                    evs.append((a, b))
+                torch.cuda.synchronize()
+                ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs[8:])
+                med = ts[len(ts) // 2]
+                res["points"].append({"pattern": label, "layer": name, "K": K, "N": N, "parts": parts,
+                                      "workgroups": (N // 256) * parts if pattern == 0 else 256, "bytes": nbytes,
+                                      "us": round(med, 2), "GBps": round(nbytes / med / 1e3, 1),
+                                      "frac_hbm": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)})
+                log(f"   stream probe {name:13s} {med:8.2f} us  {nbytes / med / 1e3:8.1f} GB/s  ({label})")
+            del contiguous, padded
         big = [torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(2)]
         evs = []
         for r in range(20):
@@ -248,7 +240,8 @@ def main():
         torch.cuda.synchronize()
         ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs[4:])
         med = ts[len(ts) // 2]
-        res["points"].append({"pattern": "linear, 1 KiB per wave instruction", "bytes": 1 << 30, "us": round(med, 2),
+        res["points"].append({"pattern": "one contiguous run per wave", "layer": "1 GiB buffer", "workgroups": 256,
+                              "bytes": 1 << 30, "us": round(med, 2),
                               "GBps": round((1 << 30) / med / 1e3, 1), "frac_hbm": round((1 << 30) / med / 1e3 / HBM_PEAK_GBS, 4)})
         log(f"   stream probe linear 1 GiB  {med:8.2f} us  {(1 << 30) / med / 1e3:8.1f} GB/s")
         print(json.dumps(res))

@@ -65,7 +65,9 @@ size_t awqmi_dev_gemm_dense_workspace_bytes(int M, int K, int N);
  * awqmi_dev_stream_probe: a read-only pass with the arithmetic removed.  pattern 0 reads an int32
  * [K, N / 8] matrix the way the skinny GEMM kernel reads qweight (workgroup = 256 columns x one
  * of `parts` K ranges, one 128-byte line per row and 16 lanes, four 32-row steps in flight per
- * wave; K % 128 == 0, N % 256 == 0, K / 128 >= 4 parts; `out` takes (N / 256) * parts * 256 words);
+ * wave; K % 128 == 0, N % 256 == 0, K / 128 >= 4 parts; `out` takes (N / 256) * parts * 256 words;
+ * total_bytes, when not 0, is the row pitch in words of a row-padded matrix); pattern 2 is pattern 0
+ * on a column-block-major copy of the matrix (the K x 128 bytes of every 256-column block contiguous);
  * pattern 1 reads total_bytes linearly (256 workgroups, 1 KiB per wave instruction, 16 KiB in
  * flight per wave; `out` takes 65536 words).
  * awqmi_dev_mfma_probe: 256 workgroups x 4 waves, each a bare loop of fp16 MFMAs over a 128 x 128

@@ -1213,17 +1213,23 @@ int awqmi_dev_gemm_timeline_f16(const void* x, const int32_t* qweight, const voi
   return rc;
 }
 
+static inline int ldw_or(int nw, size_t pitch_words) { return pitch_words >= (size_t)nw ? (int)pitch_words : nw; }
+
 int awqmi_dev_stream_probe(const void* src, void* out, int pattern, int K, int N, int parts, size_t total_bytes,
                            void* stream) {
   if (!src || !out) return AWQMI_NULL_POINTER;
   if (!aligned16(src) || !aligned16(out)) return AWQMI_BAD_ALIGN;
   hipStream_t st = (hipStream_t)stream;
-  if (pattern == 0) {
+  if (pattern == 0 || pattern == 2) {
     // whole 128-byte lines per column block, whole 128-row chunks, at least one chunk per wave
     if (K <= 0 || N <= 0 || K % 128 != 0 || N % 256 != 0 || parts < 1 || (K / 128) < 4 * parts) return AWQMI_BAD_SHAPE;
     if ((size_t)(N / 256) * parts > 65535u * 4u) return AWQMI_BAD_SHAPE;
-    hipLaunchKernelGGL((awq_stream_probe_kernel<0>), dim3(N / 256, parts), dim3(256), 0, st,
-                       reinterpret_cast<const uint32_t*>(src), reinterpret_cast<uint32_t*>(out), K, N / 8, parts, (size_t)0);
+    if (pattern == 0)
+      hipLaunchKernelGGL((awq_stream_probe_kernel<0>), dim3(N / 256, parts), dim3(256), 0, st,
+                         reinterpret_cast<const uint32_t*>(src), reinterpret_cast<uint32_t*>(out), K, ldw_or(N / 8, total_bytes), parts, (size_t)0);
+    else
+      hipLaunchKernelGGL((awq_stream_probe_kernel<2>), dim3(N / 256, parts), dim3(256), 0, st,
+                         reinterpret_cast<const uint32_t*>(src), reinterpret_cast<uint32_t*>(out), K, 32, parts, (size_t)0);
   } else if (pattern == 1) {
     if (total_bytes < (1u << 20) || total_bytes % 1024 != 0) return AWQMI_BAD_SHAPE;
     hipLaunchKernelGGL((awq_stream_probe_kernel<1>), dim3(256), dim3(256), 0, st, reinterpret_cast<const uint32_t*>(src),

@@ -17,16 +17,20 @@ namespace awqmi {
 // Loaded words are folded into one value per lane and stored, so nothing is optimised away.
 template <int PATTERN>
 __global__ __launch_bounds__(256, 1) void awq_stream_probe_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ out,
-                                                                  int K, int ldw, int parts, size_t total_bytes) {
+                                                                  int K, int ldw, int parts, size_t total_bytes) {  // ldw: row pitch in words
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   u2v fold = {0u, 0u};
-  if constexpr (PATTERN == 0) {
+  if constexpr (PATTERN == 0 || PATTERN == 2) {
     const int cb = blockIdx.x, part = blockIdx.y;
     const int j = lane & 15, h = lane >> 4;
     const int nchunks = K >> 7;
     const unsigned pw = (unsigned)part * 4u + (unsigned)wave, np = (unsigned)parts * 4u;
     const int c0 = (int)(pw * (unsigned)nchunks / np), c1 = (int)((pw + 1) * (unsigned)nchunks / np);
-    const char* base = reinterpret_cast<const char*>(src) + ((size_t)(8 * h) * ldw + cb * 32 + 2 * j) * 4;
+    // PATTERN 2: the same reads on a column-block-major copy of the matrix (the K x 128 bytes of a
+    // column block contiguous, rows 128 bytes apart)
+    const char* base = PATTERN == 2 ? reinterpret_cast<const char*>(src) + ((size_t)cb * K * 32 + (size_t)(8 * h) * 32 + 2 * j) * 4
+                                    : reinterpret_cast<const char*>(src) + ((size_t)(8 * h) * ldw + cb * 32 + 2 * j) * 4;
+    if (PATTERN == 2) ldw = 32;
     u2v q[4][8];
     auto issue = [&](int d, int step) {
       const char* rb = base + (size_t)step * 32 * ldw * 4;
