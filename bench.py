@@ -9,9 +9,21 @@ uses copy M, so between two uses of the same buffer ~1.8 GB of other weights str
 and the 256 MB Infinity Cache cannot serve them: the reported figure is HBM bandwidth.
 
 `value` = algorithmic bytes of a step (packed weights + scales + packed zeros + activations
-in + out) / time per step.  The prefill sweep (M in {512, 2048, 8192}, fp16 MFMA TFLOP/s) is
-measured after the timed region and reported under "prefill".  The CPU baseline leg times
-the PyTorch dequantize-then-matmul oracle on the host cores over a bounded sample.
+in + out) / time per step, timed over exactly --steps steps after exactly --warmup untimed ones.
+The chip's clocks take about 20 ms of load to settle, so the same sweep timed after at least 50
+untimed steps is reported beside it under "settled".  The dense layers' qweight is held as this
+package's layer method holds it after loading (--rows method, the path a served model takes);
+the contiguous layout's sweep is reported under "other_qweight_rows".
+
+The prefill sweep (M in {512, 2048, 8192}, fp16 MFMA TFLOP/s) is measured after the timed region
+and reported under "prefill": per point the sustained rate (at least 100 ms of back-to-back calls
+timed after at least 50 ms untimed; the chip holds a lower clock under lasting matrix load) with
+the burst rate of a few launches beside it.  The CPU baseline leg times the PyTorch
+dequantize-then-matmul oracle on the host cores over a bounded sample.
+
+--probe measures a ceiling instead (what HBM delivers for the decode kernel's access pattern,
+what the matrix pipe sustains under the power limit, where a decode launch's time goes);
+--pmc-target runs a fixed set of launches for rocprofv3 counter collection.
 
 Prints ONE JSON line on stdout; progress goes to stderr.
 """
@@ -104,7 +116,8 @@ def main():
                     help="counter-collection mode for rocprofv3 --pmc, no timing.  decode: the 16-launch "
                          "decode sweep twice (direct launches) plus four 256 MiB device copies "
                          "(calibration of FETCH_SIZE / WRITE_SIZE).  prefill: awq_gemm at o_proj, "
-                         "M=8192, three times.  moe: the Qwen3-30B-A3B MoE block at T=512, five times")
+                         "M=8192, twelve times in its default form (panel pass + dense kernel) and twelve times as "
+                         "the per-tile kernel.  moe: the Qwen3-30B-A3B MoE block at T=512, five times")
     ap.add_argument("--probe", choices=("hbm-stream", "mfma", "decode-timeline"), default=None,
                     help="measure a ceiling instead of the benchmark and print it as JSON.  hbm-stream: the skinny "
                          "kernel's weight access pattern with the arithmetic removed over the four 72B qweight "

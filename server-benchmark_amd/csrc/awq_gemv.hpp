@@ -1,16 +1,22 @@
-// Skinny AWQ GEMM (M <= 16 rows per launch block): Y[M,N] = X[M,K] @ dequant(W), HBM-bound.
+// Skinny AWQ GEMM (16 rows per row block, one or two row blocks per pass): Y[M,N] = X[M,K] @
+// dequant(W), HBM-bound.
 //
 // One wave owns a block of 128*WPL output columns and a contiguous range of 128-row chunks
 // of K.  Per 32-row step each lane loads 8 rows x WPL packed words (16 lanes side by side
-// cover 64*WPL contiguous bytes of a row, the four 16-lane groups take four 8-row slabs),
-// turns the 8x8 nibble block of every word into the B operand of v_mfma_f32_16x16x32_f16
-// with one v_perm_b32 + two v_and_or_b32 + two v_pk_add_f16 per four weights, and feeds it
-// against the 16xK activation slab (A operand, straight from global memory).  The integer
-// difference (w - z) goes through the matrix core; the group scale is applied to the
-// per-group accumulator in fp32, so no per-weight multiply is spent.  Four waves of a
-// workgroup split the workgroup's K range and meet in LDS; workgroups of a split-K launch
-// meet through fp32 partials in the workspace, summed in fixed order by whichever
-// workgroup arrives last (arrival counter per column block, left at zero).
+// cover 64*WPL contiguous bytes of a row, the four 16-lane groups take four 8-row slabs) and
+// turns the 8x8 nibble block of every word into B operands of v_mfma_f32_16x16x32_f16 without
+// converting anything: a nibble left in place in a 16-bit lane IS the fp16 subnormal w * 2^-24
+// (w * 2^-20 for the high nibble of a byte), which the matrix core takes exactly.  Per four
+// weights that is one v_perm_b32 (byte gather in AWQ nibble order) and one v_and_b32: the low
+// nibble is not masked, the whole byte goes in as (16 w' + w) * 2^-24 and the high-nibble tile's
+// sum is taken off again in fp32 when the group ends.  The operands run against the 16xK
+// activation slab (A operand, straight from global memory).  The zero point costs one 16-deep
+// MFMA per group (A = the lane's sum of activations in four fp16 pieces, B = -z * 2^-e); the
+// group scale is applied to the per-group accumulator in fp32 and 2^e once at the end, so no
+// per-weight subtract or multiply is spent.  Four waves of a workgroup split the workgroup's K
+// range and meet in LDS; workgroups of a split-K launch meet through fp32 partials in the
+// workspace, summed in fixed order by whichever workgroup arrives last (arrival counter per
+// column block, left at zero).
 #pragma once
 #include "awq_common.hpp"
 #include "awq_moe.hpp"
