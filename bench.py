@@ -117,7 +117,8 @@ def main():
                          "decode sweep twice (direct launches) plus four 256 MiB device copies "
                          "(calibration of FETCH_SIZE / WRITE_SIZE).  prefill: awq_gemm at o_proj, "
                          "M=8192, twelve times in its default form (panel pass + dense kernel) and twelve times as "
-                         "the per-tile kernel.  moe: the Qwen3-30B-A3B MoE block at T=512, five times")
+                         "the per-tile kernel.  moe: the Qwen3-30B-A3B MoE block at T=512, five times, then its w13 GEMM "
+                         "alone with 16-row and with 32-row sorted-token blocks, five times each")
     ap.add_argument("--probe", choices=("hbm-stream", "mfma", "decode-timeline"), default=None,
                     help="measure a ceiling instead of the benchmark and print it as JSON.  hbm-stream: the skinny "
                          "kernel's weight access pattern with the arithmetic removed over the four 72B qweight "
@@ -355,7 +356,17 @@ def main():
         for _ in range(5):
             sba.fused_moe_awq(xm, w13, w2, lg, topk, True)
         torch.cuda.synchronize()
-        log(f"[bench] pmc target: 5 x MoE block, T=512, {E} experts, top-{topk}, hidden {H}, inter {I}")
+        # the w13 expert GEMM alone, step by step: 16-row sorted-token blocks (what the block above uses
+        # at this size), then 32-row blocks with one packed word per lane -- for a side-by-side record of
+        # what the wider blocks do to the L2 request count
+        wts, ids = ops.topk_softmax(lg, topk, True)
+        for bs in (16, 32):
+            sorted_ids, expert_ids, npp = ops.moe_align_block_size(ids, bs, E)
+            for _ in range(5):
+                ops.moe_awq_gemm(xm, *w13, sorted_ids, expert_ids, npp, 512 * topk, topk, block_size=bs)
+        torch.cuda.synchronize()
+        log(f"[bench] pmc target: 5 x MoE block, T=512, {E} experts, top-{topk}, hidden {H}, inter {I}; then the w13 "
+            f"GEMM alone 5 x with 16-row and 5 x with 32-row blocks")
         return
     if args.pmc_target == "decode":
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)

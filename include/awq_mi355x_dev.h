@@ -29,6 +29,10 @@
  *   1 << 25  awq_gemm never takes the dequantise-once form (many-row calls run the fused kernel)
  *   1 << 26  awq_gemm takes the dequantise-once form from 257 rows on, when the workspace holds
  *            awqmi_dev_gemm_dense_workspace_bytes()
+ *   1 << 27  expert GEMMs over 32-row sorted-token blocks (tile_m = 32) in the older form with two
+ *            packed words per lane and one workgroup per CU (default for tile_m = 32 without a K
+ *            split: one word per lane, two 128-column blocks per workgroup, weight ring in LDS, two
+ *            workgroups per CU; with 4096 its ring stays in registers)
  * The workspace must be large enough for the form that is forced: the sizes the public queries
  * return cover every variant except a forced MFMA tile size, which silently runs without its K
  * split when the workspace is too small for it.

@@ -870,7 +870,10 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   const int wpl = pl.wpl, ncb = pl.ncb, nblk = pl.nblk, split = pl.split;
   // 32-row blocks: one packed word per lane, two column blocks of 128 per workgroup with two waves
   // each (the accumulators of two row blocks then take the registers one row block takes with two
-  // words per lane, and two workgroups still fit a CU); needs an even chunk count, no K split
+  // words per lane, and two workgroups still fit a CU), the weight ring of four steps in LDS;
+  // needs an even chunk count, no K split.  (One 128-column block per workgroup with four K
+  // ranges measured 35 - 70 % slower: neighbouring workgroups then fetch the two halves of every
+  // 128-byte line.)
   const bool t32_narrow = tile_m == 32 && split == 1 && (K / 128) % 2 == 0 && !variant_on(VAR_MOE_T32_WIDE);
   if (tile_m == 32 && !t32_narrow && wpl != 2) return AWQMI_BAD_SHAPE;   // the wide form needs N % 16 == 0
   if (split > 1) {
@@ -920,6 +923,7 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   p.act_split = act_split ? 1 : 0;
   const bool act_pair = fuse_act && split == 1;
   const int ncb1 = (NW + 15) / 16;       // column blocks of 128 (one word per lane)
+  const bool t32_lds = t32_narrow && (size_t)K * NW * 4 < (1ull << 31) && !variant_on(VAR_NO_LDS_RING);
   const int ncg = t32_narrow ? (ncb1 + 1) / 2 : (act_pair ? ncb / 2 : (pair_cols ? (ncb + 1) / 2 : ncb));
   if (t32_narrow) p.ncb = ncb1;
   // runs of grp slots, dealt to the 8 XCDs in turn; the last deal may be partial
@@ -960,6 +964,7 @@ static int moe_gemm_impl(const void* x, const int32_t* qweight, const void* scal
   else if (ldsq) launch_gemv<2, 1, true, 4, 4, false, true>(p, grid, st);
   else if (act_pair) launch_gemv<2, 1, true, 2, 2, true>(p, grid, st);
   else if (act_split) launch_gemv<2, 1, true, 2>(p, grid, st);
+  else if (t32_lds) launch_gemv<1, 2, true, 4, 2, false, true>(p, grid, st);
   else if (t32_narrow) launch_gemv<1, 2, true, 2, 2>(p, grid, st);
   else if (tile_m == 32) launch_gemv<2, 2, true>(p, grid, st);
   else if (wpl == 2 && variant_on(VAR_MOE_RING4)) launch_gemv<2, 1, true, 4>(p, grid, st);

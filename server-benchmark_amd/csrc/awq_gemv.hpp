@@ -127,12 +127,16 @@ struct WordVec<2> {
 // MB row blocks of 16 share every B operand (MB = 2 serves up to 32 rows per pass with the
 // unpack work of one).  GMODE: 0 -> G = 32, 1 -> G = 64, 2 -> G = 128, 3 -> G = 128 * i.
 //
-// LDSQ: the weight ring lives in LDS instead of registers.  A 32-row step of a wave is 4 KiB
-// (32 rows x 128 bytes, WPL = 2 only); four `buffer_load_dwordx4 ... lds` instructions fetch it
+// LDSQ: the weight ring lives in LDS instead of registers.  With WPL = 2 a 32-row step of a wave
+// is 4 KiB (32 rows x 128 bytes); four `buffer_load_dwordx4 ... lds` instructions fetch it
 // (lane l of instruction i brings 16 bytes of row 8 i + l / 8), and the step is read back as
-// eight 8-byte LDS loads per lane right before its compute.  Ring slot d of all waves is one
-// LDS object of its own, so that the compiler's wait before reading a slot counts only the
-// loads issued after that slot's.  This buys a ring of four steps at two waves per SIMD.
+// eight 8-byte LDS loads per lane right before its compute.  With WPL = 1 a step is 2 KiB (32 rows
+// x 64 bytes), fetched by two instructions (lane l of instruction i brings 16 bytes of row
+// 4 i + l / 16 + 8 ((l / 4) % 4), so that row 8 h + r lands in 64-byte piece 4 r + h of the slot and
+// the four 16-lane groups of a read hit four different quarters of the banks) and read back as
+// eight 4-byte LDS loads per lane.  Ring slot d of all waves is one LDS object of its own, so that
+// the compiler's wait before reading a slot counts only the loads issued after that slot's.  This
+// buys a ring of four steps at two waves per SIMD.
 //
 // TAIL (G = 128, register ring of four): after its whole chunks the wave takes one more 32-row
 // step of a chunk that the launch's waves share step by step.  When the chunk count leaves
@@ -157,7 +161,7 @@ struct GemvWave {
   qvec q[LDSQ ? 2 : RING][8];   // LDSQ: the step being computed and the next one, read from the LDS ring
   u4v a[RING][MB];
   // LDSQ only
-  unsigned char* slot[RING];      // this wave's 4 KiB in each ring slot object
+  unsigned char* slot[RING];      // this wave's 2 KiB x WPL in each ring slot object
   __amdgpu_buffer_rsrc_t rq;      // the (expert's) qweight as a buffer: loads past its end return 0
   // Row r of a step sits in 128-byte line r ^ ((r >> 3) & 1) of the slot: the two 8-row
   // blocks that one half-wave reads together then fall into different halves of the 64 banks.
@@ -175,10 +179,17 @@ struct GemvWave {
 #if defined(__HIP_DEVICE_COMPILE__)
       typedef __attribute__((address_space(3))) void lds_void;
       const uint32_t so = (uint32_t)ks * 32u * (uint32_t)LDW * 4u;
+      if constexpr (WPL == 2) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rq, (lds_void*)(slot[d] + i * 1024), 16, dma_v[i & 1],
-                                                 so + (uint32_t)i * 8u * (uint32_t)LDW * 4u, 0, 0);
+        for (int i = 0; i < 4; ++i)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rq, (lds_void*)(slot[d] + i * 1024), 16, dma_v[i & 1],
+                                                   so + (uint32_t)i * 8u * (uint32_t)LDW * 4u, 0, 0);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rq, (lds_void*)(slot[d] + i * 1024), 16, dma_v[0],
+                                                   so + (uint32_t)i * 4u * (uint32_t)LDW * 4u, 0, 0);
+      }
 #endif
     } else {
       const char* rowbase = reinterpret_cast<const char*>(qw_u) + (size_t)ks * 32 * LDW * 4;
@@ -195,8 +206,10 @@ struct GemvWave {
   // LDSQ: ring slot d -> register set d % 2
   __device__ __forceinline__ void fetch(int d) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      q[d & 1][i] = *reinterpret_cast<const qvec*>(slot[d] + rd_off[i & 1] + (i & 6) * 128);
+    for (int i = 0; i < 8; ++i) {
+      if constexpr (WPL == 2) q[d & 1][i] = *reinterpret_cast<const qvec*>(slot[d] + rd_off[i & 1] + (i & 6) * 128);
+      else q[d & 1][i] = *reinterpret_cast<const qvec*>(slot[d] + rd_off[0] + i * 256);
+    }
   }
 
   __device__ __forceinline__ int clamp_group(int step) const {
@@ -437,7 +450,8 @@ template <int WPL, int GMODE, int MB, bool MOE, int RING, int KW, bool ACT, bool
 __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
   static_assert(RPER == 0 || (MOE && MB == 1 && !TAIL), "folded routing: expert-grouped launches of 16-row blocks");
   static_assert(!ACT || (KW == 2 && MB == 1), "fused activation pairs two column blocks");
-  static_assert(!LDSQ || (WPL == 2 && RING == 4), "the LDS ring holds four steps of 128-byte rows");
+  static_assert(!LDSQ || RING == 4, "the LDS ring holds four steps");
+  static_assert(!LDSQ || WPL == 2 || (MB == 2 && KW == 2), "one word per lane in LDS: the 32-row form");
   static_assert(!TAIL || (!MOE && KW == 4 && !ACT), "tail steps are for dense launches");
   constexpr int CW = 4 / KW;       // column blocks per workgroup
   constexpr int NT = 8 * WPL;
@@ -446,7 +460,7 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
   // unpadded where the two buffers take the place of ring slots 0 and 1 (16 KiB each)
   constexpr int RS = LDSQ ? NT * 16 : NT * 16 + 4;
   constexpr int TM = 16 * MB;      // rows per pass
-  constexpr int SLOT = LDSQ ? 16384 : 16;   // bytes of one ring slot object: four waves x 4 KiB
+  constexpr int SLOT = LDSQ ? 8192 * WPL : 16;   // bytes of one ring slot object: four waves x 2 KiB x WPL
   __shared__ __align__(16) unsigned char lq0[SLOT], lq1[SLOT], lq2[SLOT], lq3[SLOT];
   __shared__ __align__(16) float red_own[LDSQ ? 1 : 2][LDSQ ? 1 : 16][RS];
   auto red = [&](int b) -> float (*)[RS] {
@@ -590,15 +604,25 @@ __device__ __forceinline__ void awq_gemv_body(const GemvParams& p) {
   if constexpr (LDSQ) {
     unsigned char* const slots[4] = {lq0, lq1, lq2, lq3};
 #pragma unroll
-    for (int d = 0; d < RING; ++d) w.slot[d] = slots[d] + wave_u * 4096;
+    for (int d = 0; d < RING; ++d) w.slot[d] = slots[d] + wave_u * (2048 * WPL);
     w.rq = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(qw), 0, (int)((size_t)p.K * p.ldw * 4), 0x00020000);
-    const int wc4 = cbw * (16 * WPL) + 4 * (lane & 7);       // first of the four words this lane fetches
-    // line 8 i + l / 8 of the slot (instruction i, lane l) holds row 8 i + ((l / 8) ^ (i & 1))
-    w.dma_v[0] = (uint32_t)(((size_t)(lane >> 3) * p.ldw + (wc4 < p.NW ? wc4 : 0)) * 4);
-    w.dma_v[1] = (uint32_t)(((size_t)((lane >> 3) ^ 1) * p.ldw + (wc4 < p.NW ? wc4 : 0)) * 4);
-    // row 8 h + i is read from line 8 h + (i ^ (h & 1))
-    w.rd_off[0] = (uint32_t)((8 * h + (h & 1)) * 128 + 8 * j);
-    w.rd_off[1] = (uint32_t)((8 * h + (1 ^ (h & 1))) * 128 + 8 * j);
+    if constexpr (WPL == 2) {
+      const int wc4 = cbw * (16 * WPL) + 4 * (lane & 7);       // first of the four words this lane fetches
+      // line 8 i + l / 8 of the slot (instruction i, lane l) holds row 8 i + ((l / 8) ^ (i & 1))
+      w.dma_v[0] = (uint32_t)(((size_t)(lane >> 3) * p.ldw + (wc4 < p.NW ? wc4 : 0)) * 4);
+      w.dma_v[1] = (uint32_t)(((size_t)((lane >> 3) ^ 1) * p.ldw + (wc4 < p.NW ? wc4 : 0)) * 4);
+      // row 8 h + i is read from line 8 h + (i ^ (h & 1))
+      w.rd_off[0] = (uint32_t)((8 * h + (h & 1)) * 128 + 8 * j);
+      w.rd_off[1] = (uint32_t)((8 * h + (1 ^ (h & 1))) * 128 + 8 * j);
+    } else {
+      const int wc4 = cbw * 16 + 4 * (lane & 3);
+      // 64-byte piece 16 i + l / 4 of the slot (instruction i, lane l) holds row 4 i + l / 16 + 8 ((l / 4) % 4)
+      w.dma_v[0] = (uint32_t)(((size_t)((lane >> 4) + 8 * ((lane >> 2) & 3)) * p.ldw + (wc4 < p.NW ? wc4 : 0)) * 4);
+      w.dma_v[1] = 0;
+      // row 8 h + i is read from piece 4 i + h
+      w.rd_off[0] = (uint32_t)(h * 64 + 4 * j);
+      w.rd_off[1] = 0;
+    }
   }
   w.q_off = (uint32_t)(((size_t)8 * h * p.ldw + wc) * 4);
   w.sc = sc + 8 * (size_t)wc;

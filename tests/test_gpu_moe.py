@@ -127,6 +127,55 @@ def test_moe_grouped_gemm_block_sizes(sba, gpu, bs):
     assert err <= TOL
 
 
+@pytest.mark.parametrize("T,E,topk,K,N,G", [
+    (37, 8, 2, 256, 264, 128),      # ragged last word column, an odd number of 128-column blocks
+    (300, 6, 2, 768, 512, 128),     # several blocks per expert, three chunks per wave
+    (97, 5, 1, 512, 384, 64),       # top-1, group 64
+    (64, 4, 2, 256, 128, 32),       # group 32, a single column block
+    (1, 4, 2, 1024, 2048, 128),     # a single token: every block is nearly all padding
+])
+@pytest.mark.parametrize("variant", [None, 4096, 1 << 27])
+def test_moe_grouped_gemm_32_row_forms(sba, gpu, T, E, topk, K, N, G, variant):
+    """32-row sorted-token blocks without a K split: one packed word per lane with the weight ring in
+    LDS (default), the same with the ring in registers (4096), and the two-words-per-lane form
+    (1 << 27, N % 16 == 0 only), against per-slot oracle products."""
+    if variant == (1 << 27) and N % 16 != 0:
+        pytest.skip("two words per lane need N % 16 == 0")
+    rng = np.random.default_rng(T + K + N)
+    w = rng.integers(0, 16, (E, K, N))
+    z = rng.integers(0, 16, (E, K // G, N))
+    s = (rng.random((E, K // G, N)) * 0.019 + 0.001).astype(np.float16)
+    qw, qz = awq_ref.pack_awq(w), awq_ref.pack_awq(z)
+    x = rng.normal(0, 1, (T, K)).astype(np.float16)
+    ids = np.stack([rng.choice(E, size=topk, replace=False) for _ in range(T)]).astype(np.int32)
+    tw = rng.random((T, topk)).astype(np.float32)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+    sid, eid, npp = sba.moe_align_block_size(t(ids), 32, E)
+    out = torch.full((T * topk, N), float("nan"), dtype=torch.float16, device=gpu)
+    y = sba.moe_awq_gemm(t(x), t(qw), t(s), t(qz), sid, eid, npp, T * topk, topk, topk_weights=t(tw),
+                         block_size=32, out=out, _dev_variant=variant).cpu().numpy()
+    assert np.all(np.isfinite(y))            # every slot row written
+    ref = np.zeros((T * topk, N))
+    for e in range(E):
+        tok, slot = np.nonzero(ids == e)
+        if tok.size:
+            ref[tok * topk + slot] = awq_ref.gemm_wide(x[tok], qw[e], s[e], qz[e], G) * tw[tok, slot][:, None]
+    err = awq_ref.rel_frobenius(y, ref)
+    print(f"[moe grouped 32-row T={T} K={K} N={N} G={G} variant={variant}] rel_fro={err:.2e}", flush=True)
+    assert err <= TOL
+    # one X row per slot (the second expert GEMM's addressing), no routing weight
+    xs = rng.normal(0, 1, (T * topk, K)).astype(np.float16)
+    y2 = sba.moe_awq_gemm(t(xs), t(qw), t(s), t(qz), sid, eid, npp, T * topk, 1, block_size=32,
+                          _dev_variant=variant).cpu().numpy()
+    ref2 = np.zeros((T * topk, N))
+    flat = ids.reshape(-1)
+    for e in range(E):
+        rows = np.nonzero(flat == e)[0]
+        if rows.size:
+            ref2[rows] = awq_ref.gemm_wide(xs[rows], qw[e], s[e], qz[e], G)
+    assert awq_ref.rel_frobenius(y2, ref2) <= TOL
+
+
 @pytest.mark.parametrize("bs,T,E,topk,K,N,G", [
     (64, 300, 6, 2, 256, 264, 128),     # ragged last column tile, ragged last blocks
     (128, 300, 6, 2, 256, 264, 128),
