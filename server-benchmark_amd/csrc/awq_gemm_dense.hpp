@@ -241,8 +241,7 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_dense_kernel(const DenseGemmP
   };
   h8 xf[2][8], wf[2][8];
 
-  // One k-step of 64 MFMAs out of fragment set FS, in 32 pairs (one weight fragment against two
-  // activation fragments).  Between the pairs go the 16 fragment reads of the next k-step (k-step
+  // One k-step of 64 MFMAs out of fragment set FS, in 32 pairs.  Between the pairs go the 16 fragment reads of the next k-step (k-step
   // KSN of tiles xr / wr, into the other fragment set) and eight direct-to-LDS loads: of the X
   // tile (WLOAD = 0) or the W tile (WLOAD = 1) of k-stage kt_load into buffer dst.  The order is
   // pinned as written: the MFMAs are asm statements, which the scheduler's instruction groups
@@ -252,12 +251,20 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_dense_kernel(const DenseGemmP
     constexpr int fs = decltype(FS)::value, ksn = decltype(KSN)::value;
 #pragma unroll
     for (int h = 0; h < 32; ++h) {
-      const int i = h >> 2, j0 = 2 * (h & 3);
-      dg_mfma(acc[i][j0], wf[fs][i], xf[fs][j0]);
-      dg_mfma(acc[i][j0 + 1], wf[fs][i], xf[fs][j0 + 1]);
+      // 2 x 2 blocks of accumulator tiles, walked so that one operand changes from one MFMA to the
+      // next (block rows run forth and back): under the power limit this order sustains 3 % more
+      // than "one weight fragment against all eight activation fragments" in a bare MFMA loop
+      const int b = h >> 1, i = 2 * (b >> 2), j = (b & 4) ? 6 - 2 * (b & 3) : 2 * (b & 3);
+      if (!(h & 1)) {
+        dg_mfma(acc[i][j], wf[fs][i], xf[fs][j]);
+        dg_mfma(acc[i + 1][j], wf[fs][i + 1], xf[fs][j]);
+      } else {
+        dg_mfma(acc[i + 1][j + 1], wf[fs][i + 1], xf[fs][j + 1]);
+        dg_mfma(acc[i][j + 1], wf[fs][i], xf[fs][j + 1]);
+      }
       __builtin_amdgcn_sched_barrier(0);
-      // at most one memory instruction per pair of MFMAs (weights first: the next k-step starts
-      // with wf[0], xf[0..1])
+      // at most one memory instruction per pair of MFMAs (the next k-step starts with wf[0..1],
+      // xf[0..1], which are read first)
       const int f = h >> 2;
       if ((h & 3) == 0) wf[fs ^ 1][f] = *reinterpret_cast<const h8*>(wr + 16 * f * DG_ROW_BYTES + fw_off[ksn]);
       else if ((h & 3) == 2) xf[fs ^ 1][f] = *reinterpret_cast<const h8*>(xr + 16 * f * DG_ROW_BYTES + fx_off[ksn]);

@@ -82,8 +82,10 @@ __global__ __launch_bounds__(256, 1) void awq_stream_probe_kernel(const uint32_t
 // SHAPE 0: v_mfma_f32_32x32x16_f16, 4 x 4 accumulator tiles per wave; SHAPE 1: v_mfma_f32_16x16x32_f16,
 // 8 x 8 tiles: the two ways to hold a 128 x 128 wave tile.  Two fragment sets of random fp16 values
 // (read once from src: 64 KiB per workgroup) alternate, so consecutive k-steps see different
-// operands as they do in a GEMM.  One iteration = 2 k-steps = 2 x 524288 flop per lane-row... i.e.
-// 2 x 128 x 128 x 32 x 2 = 2097152 flop per wave.
+// operands as they do in a GEMM; the MFMAs of a k-step run over 2 x 2 blocks of accumulator tiles so
+// that one operand changes from one instruction to the next (the order that sustains the most under
+// the power limit: 3 % over row-major, 6 % over an order that changes both operands every time).
+// One iteration = 2 k-steps = 2 x 128 x 128 x 32 x 2 = 2097152 flop per wave.
 template <int SHAPE>
 __global__ __launch_bounds__(256, 1) void awq_mfma_probe_kernel(const uint32_t* __restrict__ src, float* __restrict__ out,
                                                                 int iters) {
@@ -112,10 +114,13 @@ __global__ __launch_bounds__(256, 1) void awq_mfma_probe_kernel(const uint32_t* 
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s ^ ks][i], b[s][j], acc[i][j], 0, 0, 0);
+          for (int blk = 0; blk < 4; ++blk) {   // 2 x 2 blocks of tiles, one operand changing per MFMA
+            const int i = 2 * (blk >> 1), j = (blk & 2) ? 2 - 2 * (blk & 1) : 2 * (blk & 1);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s ^ ks][i], b[s][j], acc[i][j], 0, 0, 0);
+            acc[i + 1][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s ^ ks][i + 1], b[s][j], acc[i + 1][j], 0, 0, 0);
+            acc[i + 1][j + 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s ^ ks][i + 1], b[s][j + 1], acc[i + 1][j + 1], 0, 0, 0);
+            acc[i][j + 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s ^ ks][i], b[s][j + 1], acc[i][j + 1], 0, 0, 0);
+          }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -141,10 +146,13 @@ __global__ __launch_bounds__(256, 1) void awq_mfma_probe_kernel(const uint32_t* 
 #pragma unroll
       for (int s = 0; s < 2; ++s)
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-            asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(a[s][i]), "v"(b[s][j]));
+        for (int blk = 0; blk < 16; ++blk) {    // the dense GEMM kernel's order: 2 x 2 blocks of tiles, block rows forth and back
+          const int i = 2 * (blk >> 2), j = (blk & 4) ? 6 - 2 * (blk & 3) : 2 * (blk & 3);
+          asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(a[s][i]), "v"(b[s][j]));
+          asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i + 1][j]) : "v"(a[s][i + 1]), "v"(b[s][j]));
+          asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i + 1][j + 1]) : "v"(a[s][i + 1]), "v"(b[s][j + 1]));
+          asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j + 1]) : "v"(a[s][i]), "v"(b[s][j + 1]));
+        }
     }
     asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
 #pragma unroll
