@@ -585,7 +585,7 @@ def main():
                                     "this load than in its first milliseconds); TFLOPs_burst = 3 - 6 launches after two "
                                     "warm-up launches; aggregate = total flops / total time over the 12 points",
                           "kernels": "awq_gemm_mfma_kernel (fused) below 2048 rows; awq_dequant_panel_kernel + "
-                                     "awq_gemm_dense_kernel from 2048 rows on (the panel pass is inside the timed call)",
+                                     "awq_gemm_dense_kernel from 2048 rows on these layers (the panel pass is inside the timed call)",
                           "points": pts}
         log(f"[bench] prefill sweep aggregate {agg:.1f} TFLOP/s sustained ({agg / MFMA_FP16_PEAK_TFLOPS:.1%} of fp16 MFMA "
             f"peak), {agg_burst:.1f} burst")

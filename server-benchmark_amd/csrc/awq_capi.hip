@@ -230,13 +230,21 @@ MfmaPlan plan_mfma(int M, int K, int N, int bm) {
 // an fp16 panel in the workspace, then awq_gemm_dense_kernel.  Under sustained load on the 72B
 // layer shapes (fused kernel against panel pass + dense kernel, timed in turn): 512 rows 0.70,
 // 1024 rows 0.79 - 0.90, 2048 rows 1.01 - 1.03, 3072 rows 1.01 - 1.07, 4096 rows 1.08, 8192 rows
-// 1.11 - 1.16 of the fused kernel's rate; so it is taken from 2048 rows on.  K % 64 == 0 and
-// G % 8 == 0 (both implied by the MFMA path's conditions).
+// 1.11 - 1.16 of the fused kernel's rate; so it is taken from 2048 rows on.  Between 2048 and
+// 4095 rows only when the 256 x 256 tiles make at least three quarters of a round of workgroups:
+// with fewer the fused kernel's smaller row tiles fill the chip better (layers of 7B ... 32B-class
+// models at 2048 rows: 0.90 - 0.99 with 64 - 160 tiles, 1.02 - 1.08 from 224 tiles on; at 4096 rows
+// 0.98 - 1.16, at 8192 rows 1.14 - 1.21 whatever the tile count).  K % 64 == 0 and G % 8 == 0 (both
+// implied by the MFMA path's conditions).
 constexpr int DENSE_MIN_ROWS = 2048;
-inline bool dense_rows(int M) {
+inline bool dense_default(int M, int N) {
+  if (M < DENSE_MIN_ROWS) return false;
+  return M >= 2 * DENSE_MIN_ROWS || (long long)((M + 255) / 256) * ((N + 255) / 256) >= 192;
+}
+inline bool dense_rows(int M, int N) {
   if (variant_on(VAR_NO_DENSE)) return false;
   if (variant_on(VAR_DENSE)) return M > 256;
-  return M >= DENSE_MIN_ROWS;
+  return dense_default(M, N);
 }
 // workspace of the dequantise-once form: counters, K-split partial tiles, then the panel
 inline size_t dense_panel_offset(size_t part_bytes) {
@@ -469,7 +477,7 @@ size_t awqmi_gemm_workspace_bytes(int M, int K, int N, int split_k) {
       if (M % slab) mfma = std::max(mfma, plan_mfma(M % slab, K, N, mfma_pick_rows(M % slab, K, N)).part_bytes);
       // the dequantise-once form of many-row calls: 256-row tiles, and the fp16 panel behind the
       // partial tiles (a call with a smaller workspace runs the fused kernel instead)
-      if (M >= DENSE_MIN_ROWS) {
+      if (dense_default(M, N)) {
         size_t part = plan_mfma(slab, K, N, 256).part_bytes;
         if (M % slab) part = std::max(part, plan_mfma(M % slab, K, N, 256).part_bytes);
         const size_t dense = dense_panel_offset(part) + dg_panel_bytes(K, N) - AWQMI_WS_COUNTER_BYTES;
@@ -570,7 +578,7 @@ int awqmi_gemm_ld_f16(const void* x, const int32_t* qweight, int ldw, const void
     const int slab = mfma_slab_rows(M, K);
     // many rows: dequantise once into the workspace, then the dense kernel (same bits as the fused
     // kernel with 256-row tiles); needs the workspace to hold the panel
-    if (dense_rows(M) && workspace && aligned16(workspace)) {
+    if (dense_rows(M, N) && workspace && aligned16(workspace)) {
       size_t part = plan_mfma(slab < M ? slab : M, K, N, 256).part_bytes;
       if (M % slab) part = std::max(part, plan_mfma(M % slab, K, N, 256).part_bytes);
       const size_t panel_off = dense_panel_offset(part);

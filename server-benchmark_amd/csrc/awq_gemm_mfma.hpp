@@ -280,12 +280,26 @@ __global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const 
     for (int j = 0; j < NJ; ++j)
       bf[fs][j] = *reinterpret_cast<const h8*>(bs + 32 * j * PF_ROW_BYTES + f_off[ks ^ (2 * (j & 1))]);
   };
+  // 2 x 2 blocks of accumulator tiles, block rows walked forth and back, so that one operand
+  // changes from one MFMA to the next: the order that sustains the most under the power limit
   auto mfma_step = [&](int fs) {
+    auto one = [&](int i, int j) {
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[fs][i], bf[fs][j], acc[i][j], 0, 0, 0);
+    };
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
+    for (int bi = 0; bi < (MI + 1) / 2; ++bi) {
+      const int i = 2 * bi;
 #pragma unroll
-      for (int j = 0; j < NJ; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[fs][i], bf[fs][j], acc[i][j], 0, 0, 0);
+      for (int bb = 0; bb < (NJ + 1) / 2; ++bb) {
+        const int j = (bi & 1) ? 2 * ((NJ + 1) / 2 - 1 - bb) : 2 * bb;
+        one(i, j);
+        if (i + 1 < MI) one(i + 1, j);
+        if (j + 1 < NJ) {
+          if (i + 1 < MI) one(i + 1, j + 1);
+          one(i, j + 1);
+        }
+      }
+    }
   };
 
   // Interleave recipe for one phase of 16 MFMAs: an MFMA occupies the matrix pipe for eight

@@ -394,6 +394,15 @@ def test_gemm_dequantise_once_default_rule_and_small_workspace(sba, gpu):
     assert torch.equal(y, y_small)
     ref = awq_ref.gemm_wide(x[:64], qw, s, qz, G)
     assert awq_ref.rel_frobenius(y[:64].cpu().numpy(), ref) <= TOL
+    # the same row count on a narrow layer (64 tiles of 256 x 256): the fused kernel's smaller row tiles
+    # fill the chip better, so the default stays with it; from 4096 rows on the form is taken again
+    for rows, form in ((2048, _lib.FORM_FUSED), (4096, _lib.FORM_DENSE)):
+        xn, qwn, sn, qzn = _np_case(rows, K, 2048, G, seed=12)
+        xnd, qwnd, snd, qznd = _dev(gpu, xn, qwn, sn, qzn)
+        yn = sba.awq_gemm(xnd, qwnd, snd, qznd, 0)
+        assert lib.awqmi_dev_last_gemm_form() == form
+        refn = awq_ref.gemm_wide(xn[-64:], qwn, sn, qzn, G)
+        assert awq_ref.rel_frobenius(yn[-64:].cpu().numpy(), refn) <= TOL
 
 
 @pytest.mark.parametrize("M,K,N,G", [(3, 96, 40, 32), (20, 100, 16, 50), (2, 24, 8, 8)])

@@ -210,6 +210,9 @@ def test_workspace_and_split_k_queries(lib):
     assert lib.awqmi_gemm_workspace_bytes(8192, 8192, 8192, 0) == 65536 + 8192 * 8192 * 2
     assert lib.awqmi_gemm_workspace_bytes(4096, 8192, 8192 + 8, 0) >= 65536 + 8192 * (8192 + 256) * 2
     assert lib.awqmi_dev_gemm_dense_workspace_bytes(8192, 8192, 8192) == 65536 + 8192 * 8192 * 2
+    # 2048 .. 4095 rows on a narrow layer (fewer than 192 tiles of 256 x 256): the fused kernel, no panel
+    assert lib.awqmi_gemm_workspace_bytes(2048, 4096, 2048, 0) == 65536 + 64 * 4 * 256 * 256 * 4   # K-split partials only
+    assert lib.awqmi_gemm_workspace_bytes(4096, 4096, 2048, 0) == lib.awqmi_dev_gemm_dense_workspace_bytes(4096, 4096, 2048)
     assert lib.awqmi_dev_gemm_dense_workspace_bytes(300, 1000, 512) == 0    # K no multiple of 64
     assert lib.awqmi_gemm_workspace_bytes(512, 8192, 8192, 0) == 65536 + 64 * 4 * 256 * 256 * 4   # K split
     assert lib.awqmi_gemm_auto_split_k(512, 8192, 8192, 128) == 1
