@@ -29,7 +29,8 @@
 // power limit: a bare loop of it holds 2.0 GHz with random operands where the 32 x 32 x 16 shape
 // holds 1.6 GHz (1.78 against 1.65 PFLOP/s sustained).  The weights are the A operand and the
 // activations the B operand, so that a lane's four accumulator values of a tile are four
-// consecutive output columns of one row (8-byte stores).  Per stage a wave issues 128 MFMAs,
+// consecutive output columns of one row (8 bytes; they are gathered into whole 256-byte row
+// pieces through LDS before they are stored).  Per stage a wave issues 128 MFMAs,
 // 32 fragment reads, 16 direct-to-LDS loads and one barrier.
 #pragma once
 #include <type_traits>
@@ -352,17 +353,36 @@ __global__ __launch_bounds__(256, 1) void awq_gemm_dense_kernel(const DenseGemmP
     return;   // summed and written out by awq_gemm_dense_reduce_kernel, launched behind this kernel
   }
 
-  const int col_l = 4 * (lane >> 4), row_l = lane & 15;
+  // Output.  A lane's four values of an accumulator tile are 8 bytes of one row; stored like that,
+  // a store instruction carries sixteen 32-byte pieces, and when all workgroups finish their tiles
+  // together the write path takes 8 - 9 us per tile for them.  So the wave's 128 x 128 results go
+  // through its own 32 KiB of LDS first (every wave has read its last fragments by then: the
+  // barrier) -- row = 256 bytes, 16-byte chunk c of row r kept at chunk c ^ (r % 16), which makes
+  // the 8-byte writes of a half-wave and the 16-byte reads conflict-free -- and leave sixteen rows
+  // at a time as 16 bytes per lane, 256 contiguous bytes per row (1 % faster at K = 8192, 4 % at
+  // K = 2048, same bits).
+  dg_wait_and_barrier<0>();
+  unsigned char* const st = wave == 0 ? tb0 : (wave == 1 ? tb1 : (wave == 2 ? tb2 : tb3));
+  const int r_l = lane & 15, g = lane >> 4;
+  unsigned char* const wbase = st + r_l * 256 + 8 * (g & 1);
+  const unsigned char* const rbase = st + g * 256;
+  const int c16 = lane & 15;
+  const int col = n0 + wn + 8 * c16;      // N % 8 == 0: the eight columns are all inside or all outside
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    const int row = m0 + wm + 16 * j + row_l;
-    if (row >= p.M) continue;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int col = n0 + wn + 16 * i + col_l;      // N % 8 == 0: the four columns are all inside or all outside
-      if (col >= p.N) continue;
       const h4 v = {(half_t)acc[i][j][0], (half_t)acc[i][j][1], (half_t)acc[i][j][2], (half_t)acc[i][j][3]};
-      *reinterpret_cast<h4*>(p.y + (size_t)row * p.N + col) = v;
+      const int c = 2 * i + (g >> 1);
+      *reinterpret_cast<h4*>(wbase + 16 * j * 256 + ((c ^ r_l) << 4)) = v;
+    }
+    // rows 16 j .. 16 j + 15 of the wave's block are complete (this wave alone wrote them)
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int row = 16 * j + 4 * it + g;
+      const u4v v = *reinterpret_cast<const u4v*>(rbase + (16 * j + 4 * it) * 256 + ((c16 ^ (row & 15)) << 4));
+      const int grow = m0 + wm + row;
+      if (grow < p.M && col < p.N) *reinterpret_cast<u4v*>(p.y + (size_t)grow * p.N + col) = v;
     }
   }
 }
