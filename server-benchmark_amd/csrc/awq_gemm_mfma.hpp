@@ -283,8 +283,10 @@ __global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const 
   // 2 x 2 blocks of accumulator tiles, block rows walked forth and back, so that one operand
   // changes from one MFMA to the next: the order that sustains the most under the power limit
   auto mfma_step = [&](int fs) {
+    // the weights are the A operand and the activations the B operand, so that a lane's values of
+    // a tile are runs of four consecutive output columns of one row
     auto one = [&](int i, int j) {
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[fs][i], bf[fs][j], acc[i][j], 0, 0, 0);
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[fs][j], af[fs][i], acc[i][j], 0, 0, 0);
     };
 #pragma unroll
     for (int bi = 0; bi < (MI + 1) / 2; ++bi) {
@@ -419,26 +421,51 @@ __global__ __launch_bounds__(64 * NWV, NWV / 4) void awq_gemm_mfma_kernel(const 
     return;
   }
 
-  // D[i][j] of a 32x32 tile: j = lane % 32, i = 8 * (r / 4) + 4 * (lane / 32) + r % 4
-  const int col_l = lane & 31, row_l = 4 * (lane >> 5);
+  // Output.  acc[i][j][r] is row wm + 32 i + lane % 32, column wn + 32 j + 8 (r / 4) + 4 (lane / 32)
+  // + r % 4 of the workgroup tile: a lane holds 8-byte runs of a row.  They go through the wave's own
+  // piece of LDS (every wave has read its last fragments: the barrier) and leave as 16 bytes per
+  // lane, 64 NJ contiguous bytes per row -- stored directly, every instruction would carry 32
+  // separate 8-byte pieces.  LDS row = 64 NJ bytes, 16-byte chunk c of row r kept at chunk
+  // c ^ (r % 16) (NJ = 4) or c ^ ((r / 2) % 8) (NJ = 2): reads are conflict-free, the writes of rows
+  // r and r + 16 share banks (two passes).
+  __syncthreads();
+  constexpr int RB = 64 * NJ;                         // bytes per staged row
+  constexpr int CPR = RB / 16;                        // 16-byte chunks per row (16 or 8)
+  constexpr int RPI = 64 / CPR;                       // rows per read instruction (4 or 8)
+  unsigned char* const st = smem_raw + wave * (32 * MI * RB);
+  const int wr = lane & 31, wh = lane >> 5;
+  const int wswz = NJ == 4 ? (wr & 15) : ((wr >> 1) & 7);
+  const int rc = lane % CPR, rr0 = lane / CPR;
+  const int col = n0 + wn + 8 * rc;                   // N % 8 == 0: a chunk is all inside or all outside
 #pragma unroll
-  for (int i = 0; i < MI; ++i)
+  for (int i = 0; i < MI; ++i) {
+    float tw = 1.f;
+    if (GROUPED) tw = s_tw[wm + 32 * i + wr];
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int col = n0 + wn + 32 * j + col_l;
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const h4 v = {(half_t)(acc[i][j][4 * rg] * tw), (half_t)(acc[i][j][4 * rg + 1] * tw),
+                      (half_t)(acc[i][j][4 * rg + 2] * tw), (half_t)(acc[i][j][4 * rg + 3] * tw)};
+        const int c = 4 * j + rg;
+        *reinterpret_cast<h4*>(st + (32 * i + wr) * RB + ((c ^ wswz) << 4) + 8 * wh) = v;
+      }
+    // rows 32 i .. 32 i + 31 of the wave's block are complete (this wave alone wrote them)
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it) {
+      const int lr = 32 * i + RPI * it + rr0;
+      const int rswz = NJ == 4 ? (lr & 15) : ((lr >> 1) & 7);
+      const u4v v = *reinterpret_cast<const u4v*>(st + lr * RB + ((rc ^ rswz) << 4));
       if (col >= p.N) continue;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int lrow = wm + 32 * i + 8 * (r >> 2) + row_l + (r & 3);
-        if (GROUPED) {
-          const int sid = s_sid[lrow];
-          if (sid < p.n_slots) p.y[(size_t)sid * p.N + col] = (half_t)(acc[i][j][r] * s_tw[lrow]);
-        } else {
-          const int row = m0 + lrow;
-          if (row < p.M) p.y[(size_t)row * p.N + col] = (half_t)acc[i][j][r];
-        }
+      if (GROUPED) {
+        const int sid = s_sid[wm + lr];
+        if (sid < p.n_slots) *reinterpret_cast<u4v*>(p.y + (size_t)sid * p.N + col) = v;
+      } else {
+        const int row = m0 + wm + lr;
+        if (row < p.M) *reinterpret_cast<u4v*>(p.y + (size_t)row * p.N + col) = v;
       }
     }
+  }
 }
 
 // Sum of the split-K partial tiles.  Partial layout per (tile, part): [q][thread] groups of
@@ -461,7 +488,7 @@ __global__ __launch_bounds__(64 * NWV) void awq_gemm_mfma_reduce_kernel(const Mf
   const int nt_i = (nid % gsize) / gm;
   const int m0 = mt_i * (64 * MI), n0 = nt_i * PF_BN;
   const int wm = (wave / (NWV / 2)) * (32 * MI), wn = (wave % (NWV / 2)) * (32 * NJ);
-  const int col_l = lane & 31, row_l = 4 * (lane >> 5);
+  const int row_l = lane & 31;
   const float* tile_base = p.sk_part + (size_t)tl * p.sk_split * PF_SK_SLOT_FLOATS;
   f4 v[QPW];
 #pragma unroll
@@ -475,17 +502,34 @@ __global__ __launch_bounds__(64 * NWV) void awq_gemm_mfma_reduce_kernel(const Mf
 #pragma unroll
     for (int u = 0; u < QPW; ++u) v[u] += t[u];
   }
+  // The four groups of a thread are columns 8 rg + 4 (lane / 32) + 0..3, rg = 0..3, of one row of one
+  // 32 x 32 accumulator tile (see the producer's output comment; q0 is a multiple of four): lane l
+  // and lane l ^ 32 hold the two interleaved halves of 32 consecutive columns.  They trade two groups
+  // each, so that the lower lane stores columns 0..15 and the upper one columns 16..31 as 32 bytes.
+  static_assert(QPW == 4, "one accumulator tile row per thread");
+  const int ij = q0 >> 2;
+  const bool upper = lane >= 32;
+  u2v hv[4];
 #pragma unroll
-  for (int u = 0; u < QPW; ++u) {
-    const int q = q0 + u;
-    const int ij = q >> 2, r = (q & 3) * 4;
-    const int col = n0 + wn + 32 * (ij % NJ) + col_l;
-    const int row = m0 + wm + 32 * (ij / NJ) + 8 * (r >> 2) + row_l;
-    if (col < p.N) {
+  for (int u = 0; u < 4; ++u) {
+    const h4 o = {(half_t)v[u][0], (half_t)v[u][1], (half_t)v[u][2], (half_t)v[u][3]};
+    hv[u] = __builtin_bit_cast(u2v, o);
+  }
+  u2v got[2];
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (row + e < p.M) p.y[(size_t)(row + e) * p.N + col] = (half_t)v[u][e];
-    }
+  for (int k = 0; k < 2; ++k) {
+    const u2v give = upper ? hv[k] : hv[2 + k];
+    got[k][0] = (uint32_t)__shfl_xor((int)give[0], 32, 64);
+    got[k][1] = (uint32_t)__shfl_xor((int)give[1], 32, 64);
+  }
+  // lower lane: own 0, partner's 0, own 1, partner's 1; upper lane: partner's 2, own 2, partner's 3, own 3
+  const u4v lo = upper ? u4v{got[0][0], got[0][1], hv[2][0], hv[2][1]} : u4v{hv[0][0], hv[0][1], got[0][0], got[0][1]};
+  const u4v hi = upper ? u4v{got[1][0], got[1][1], hv[3][0], hv[3][1]} : u4v{hv[1][0], hv[1][1], got[1][0], got[1][1]};
+  const int col = n0 + wn + 32 * (ij % NJ) + (upper ? 16 : 0);
+  const int row = m0 + wm + 32 * (ij / NJ) + row_l;
+  if (row < p.M) {        // N % 8 == 0: eight columns are all inside or all outside
+    if (col < p.N) *reinterpret_cast<u4v*>(p.y + (size_t)row * p.N + col) = lo;
+    if (col + 8 < p.N) *reinterpret_cast<u4v*>(p.y + (size_t)row * p.N + col + 8) = hi;
   }
 }
 
