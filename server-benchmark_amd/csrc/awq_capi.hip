@@ -1013,10 +1013,11 @@ constexpr int MOE_ALIGN_SPLIT_MIN = 16384;   // slots from which it is used (409
 // three expert shapes (2048/768 x 128 experts, 6144/2560 x 160, 4096/14336 x 8):
 //   skinny: flops / (540 TFLOP/s * avg / (avg + 26)), avg = slots per expert;
 //   MFMA:   per GEMM blocks * column tiles / 256 CUs rounds (a partial last round counts as
-//           at least half) of (K / 64 + overhead) k-tiles at 5.7 ns * (rows + 96) each, plus
+//           at least half) of (K / 64 + overhead) k-tiles at 5.4 ns * (rows + 112) each, plus
 //           the separate SiLU pass at 4 TB/s; blocks is the expected block count after
 //           padding each expert's run to whole blocks (slots spread evenly over the experts).
-// Within 2 % of the best forced block size on 18 points over six expert shapes.
+// Within 5 % of the best forced block size on 25 points over six expert shapes (fit) and on the
+// points of three further shapes it was then checked on.
 // The MFMA form also needs every operand under 4 GiB (32-bit buffer offsets).
 int moe_pick_tile(int n_slots, int E, int H, int inter, int group) {
   if (variant_on(VAR_MOE_TILE16)) return 16;
@@ -1040,8 +1041,8 @@ int moe_pick_tile(int n_slots, int E, int H, int inter, int group) {
     for (int j = 1; j * (double)bm < avg + 6.0 * std::sqrt(avg) + 1.0; ++j)
       per_expert += 0.5 * std::erfc((j * (double)bm + 0.5 - avg) / std::sqrt(2.0 * avg));
     const double blocks = E * per_expert;
-    const double kt_s = 5.7e-9 * (bm + 96);
-    const int over = bm == 256 ? 10 : 6;
+    const double kt_s = 5.4e-9 * (bm + 112);
+    const int over = bm == 256 ? 6 : 4;
     auto gemm = [&](int K, int N) {
       const double r = blocks * ((N + PF_BN - 1) / PF_BN) / 256.0;
       const double whole = std::floor(r), part = r - whole;

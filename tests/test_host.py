@@ -181,7 +181,8 @@ def test_fused_moe_block_rows(lib):
     q = lib.awqmi_fused_moe_block_rows
     for T in (1, 16, 128, 512, 1024, 2048):
         assert q(T, 2048, 768, 128, 8, 128) == 16
-    assert q(8192, 2048, 768, 128, 8, 128) == 128
+    assert q(3072, 2048, 768, 128, 8, 128) == 256
+    assert q(8192, 2048, 768, 128, 8, 128) == 256
     assert q(512, 6144, 2560, 160, 8, 128) == 16
     assert q(1024, 6144, 2560, 160, 8, 128) == 64
     assert q(1024, 2048, 1408, 64, 6, 128) == 128
