@@ -21,6 +21,10 @@
 // Workgroup ids are spread over the eight XCDs in contiguous ranges and walked in
 // 8-row-tile groups so that the 32 workgroups resident on one XCD share X and W tiles
 // through that XCD's L2.
+//
+// The weights are the MFMA's A operand and the activations its B operand: a lane's results of a
+// tile are then 8-byte runs of an output row, which are gathered through LDS into 16 bytes per
+// lane and stored as whole row pieces.
 #pragma once
 #include "awq_common.hpp"
 
