@@ -27,7 +27,7 @@
 // Workgroup tile 256 x 256, four waves 2 x 2, each 128 x 128 = 8 x 8 v_mfma_f32_16x16x32_f16
 // accumulators.  The 16 x 16 x 32 shape is the one that gives the most flops under the chip's
 // power limit: a bare loop of it holds 2.0 GHz with random operands where the 32 x 32 x 16 shape
-// holds 1.6 GHz (1.78 against 1.65 PFLOP/s sustained).  The weights are the A operand and the
+// holds 1.7 GHz (about 1.95 against 1.7 PFLOP/s sustained).  The weights are the A operand and the
 // activations the B operand, so that a lane's four accumulator values of a tile are four
 // consecutive output columns of one row (8 bytes; they are gathered into whole 256-byte row
 // pieces through LDS before they are stored).  Per stage a wave issues 128 MFMAs,
