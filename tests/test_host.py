@@ -597,3 +597,19 @@ def test_plugin_entry_point_resolves_from_the_mounted_layout(sba):
     plugin = __import__("importlib").import_module(sba.__name__ + ".vllm_plugin")
     assert fn is plugin.register
     assert os.path.exists(os.path.join(ROOT, "server_benchmark_amd.py"))      # the alias the entry point names
+
+
+def test_bench_is_for_one_gpu_and_has_no_cpu_path():
+    """`bench.py --gpus N` with N above one exits with a message that says so; without a GPU the
+    run fails loudly instead of measuring anything on the CPU."""
+    import subprocess
+    import sys
+    bench = os.path.join(ROOT, "bench.py")
+    res = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 2 and "one GPU only" in res.stderr and res.stdout.strip() == ""
+    import torch
+    if not torch.cuda.is_available():
+        res = subprocess.run([sys.executable, bench, "--steps", "1", "--warmup", "0"], capture_output=True, text=True,
+                             timeout=300)
+        assert res.returncode == 1 and "no CPU fallback" in res.stderr and res.stdout.strip() == ""
+
