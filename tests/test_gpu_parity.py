@@ -405,6 +405,38 @@ def test_gemm_dequantise_once_default_rule_and_small_workspace(sba, gpu):
         assert awq_ref.rel_frobenius(yn[-64:].cpu().numpy(), refn) <= TOL
 
 
+def test_gemm_dequantise_once_form_replays_from_a_graph(sba, gpu):
+    """The many-row form is three plain launches (panel pass, dense kernel, K-split sum) on the
+    caller's stream and workspace: captured once, every replay -- with new activations and with
+    eager calls of other shapes on the same stream in between -- equals the eager result."""
+    from server_benchmark_amd import _lib
+    lib = _lib.load()
+    M, K, N, G = 2304, 320, 1032 * 8, 64          # 9 x 33 tiles: a sparse last round, split in K; ragged N
+    x, qw, s, qz = _np_case(M, K, N, G, seed=21)
+    xd, qwd, sd, qzd = _dev(gpu, x, qw, s, qz)
+    st = torch.cuda.Stream()
+    st.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(st):
+        eager = sba.awq_gemm(xd, qwd, sd, qzd, 0)            # sizes this stream's workspace
+        assert lib.awqmi_dev_last_gemm_form() == _lib.FORM_DENSE
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            y = sba.awq_gemm(xd, qwd, sd, qzd, 0)
+        for rep in range(3):
+            if rep:
+                xd.copy_(torch.randn((M, K), device=gpu, generator=torch.Generator(device=gpu).manual_seed(rep)).half())
+                eager = sba.awq_gemm(xd, qwd, sd, qzd, 0)
+            sba.awq_gemm(xd[:5], qwd, sd, qzd, 0)           # a skinny call on the same workspace in between
+            y.zero_()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, eager)
+    torch.cuda.current_stream().wait_stream(st)
+    ref = awq_ref.gemm_wide(xd[:32].cpu().numpy(), qw, s, qz, G)
+    assert awq_ref.rel_frobenius(y[:32].cpu().numpy(), ref) <= TOL
+
+
 @pytest.mark.parametrize("M,K,N,G", [(3, 96, 40, 32), (20, 100, 16, 50), (2, 24, 8, 8)])
 def test_gemm_generic_fallback(sba, gpu, M, K, N, G):
     x, qw, s, qz = _np_case(M, K, N, G, seed=5)
